@@ -1,0 +1,148 @@
+// The dispatch policy of the scheduler as a pure state machine.
+//
+// Everything the policy observes (queue heads, event completion, stop
+// acknowledgements, wall time) and everything it does (dispatch, release an
+// iteration, raise a stop) goes through PolicyHost, so the same code runs
+// against the live HIP runtime (scheduler/), against a recorded observation log
+// (replay.cpp) and under test.  No HIP header is needed here.
+//
+// Restates, for gfx950, the policy of the reference scheduler:
+//   src/scheduler/scheduler_eval.cpp:238-487  busy_wait_profile (Orion policy)
+//   src/scheduler/scheduler_eval.cpp:93-165   schedule_reef
+//   src/scheduler/scheduler_eval.cpp:167-236  schedule_sequential
+//   src/scheduler/utils_sched.cpp:239-522     schedule_kernel bookkeeping
+//   src/scheduler/scheduler_eval.cpp:498-540  profile parsing, setup_change
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace orion {
+
+// Record classes as the policy tells them apart.  Every library-op record is
+// kernel-like (reference: enum func_type, cuda_capture/intercept_temp.h:642-660).
+enum RecClass : int {
+  REC_NONE = -1,
+  REC_KERNEL = 0,
+  REC_MEMCPY = 1,
+  REC_MALLOC = 2,
+  REC_FREE = 3,
+  REC_MEMSET = 4,
+};
+
+inline bool is_mem_class(int c) { return c >= REC_MEMCPY && c <= REC_MEMSET; }
+char rec_class_char(int c);           // 'k','c','m','f','s'
+int rec_class_from_char(char ch);     // REC_NONE for '.', -2 for '-', -3 bad
+
+enum Algo : int { ALGO_ORION = 0, ALGO_REEF = 1, ALGO_SEQUENTIAL = 2 };
+const char* algo_name(int algo);
+int algo_from_name(const std::string& name);  // -1 if unknown
+
+// One profile row (reference: struct op_info, scheduler/utils_sched.h:90-98).
+struct OpInfo {
+  std::string name;
+  int profile;     // 1 compute-bound, 0 memory-bound, -1 unknown
+  int mem;
+  int sm_used;     // compute units the op can occupy
+  float duration;  // nanoseconds, fp32 like the reference
+};
+
+// Parses a profile CSV (header line, then Name,Profile,Memory_footprint,
+// SM_usage,Duration).  Field conversion follows std::stoi / std::stof.
+// Returns false and fills *err on an unreadable file or a malformed row.
+bool parse_profile(const std::string& path, std::vector<OpInfo>* ops,
+                   std::string* err);
+
+// CU-mask placement of a best-effort kernel: index of the smallest mask (sizes
+// ascending, last = whole GPU) that holds the op's CU need.  No reference
+// counterpart (the reference owns one stream per client).
+int place_cu_slot(const std::vector<int>& masks, int rec_class, int sm_used,
+                  int algo);
+
+struct Dispatch {
+  int client;      // whose record
+  int owner;       // whose stream / event array it goes to
+  int rec_class;
+  int op_index;    // profile row used (seen[client] before the dispatch)
+  int event_slot;  // event_ids[owner] before the dispatch
+  int cu_slot;     // CU-mask slot of the owner's stream set, -1 = unchanged
+};
+
+class PolicyHost {
+ public:
+  virtual ~PolicyHost() {}
+  virtual void begin_poll() {}
+  virtual void end_poll(bool /*effective*/) {}
+  virtual bool stop_ack(int client) = 0;
+  virtual int peek(int client) = 0;  // RecClass of the queue head or REC_NONE
+  virtual bool event_done(int owner, int index) = 0;
+  virtual int64_t iteration_us(int client) = 0;
+  virtual void dispatch(const Dispatch& d) = 0;
+  virtual void iteration_done(int client, int iteration) = 0;
+  virtual void set_stop(int client) = 0;
+};
+
+struct ScheduleArgs {
+  bool warmup = false;
+  int warmup_iters = 0;
+  int algo = ALGO_ORION;
+  int depth = 1;         // REEF queue depth, or Orion's best-effort budget (ns)
+  int hp_limit = 1;      // tolerated high-priority training iteration (ms)
+  int update_start = 1;  // first kernel of the optimizer-update phase
+  int64_t max_polls = -1;  // >= 0: give up after that many polls (tests)
+};
+
+class Policy {
+ public:
+  // max_sms: compute units of the device (80 in the reference, 256 on MI355X).
+  // sequential_fix: let the time-slicing policy dispatch when no other client
+  // is mid-iteration; the reference text can never dispatch past warm-up.
+  Policy(std::vector<std::vector<OpInfo>> profiles,
+         std::vector<int> num_kernels, std::vector<int> num_iters,
+         std::vector<bool> is_train, int max_sms,
+         std::vector<int> cu_masks, bool sequential_fix);
+
+  void setup_change(int client, std::vector<OpInfo> ops, int num_kernels);
+
+  // Runs the poll loop until every client has finished.  Returns the number
+  // of polls, or -1 when max_polls ran out first.
+  int64_t schedule(PolicyHost& host, const ScheduleArgs& args);
+
+  int num_clients() const { return n_; }
+  const std::vector<int>& cur_iters() const { return cur_iters_; }
+  const std::vector<int>& seen() const { return seen_; }
+  const std::vector<OpInfo>& ops(int client) const { return ops_[client]; }
+  int sm_threshold() const { return sm_threshold_; }
+  bool large_found() const { return large_found_; }
+  long sum() const { return sum_; }
+
+ private:
+  void dispatch(PolicyHost& host, int client, int owner, int rec_class);
+  void reef(PolicyHost& host, const std::vector<int>& heads, int depth);
+  int sequential(PolicyHost& host, const std::vector<int>& heads, int start);
+
+  int n_;
+  std::vector<std::vector<OpInfo>> ops_;
+  std::vector<int> max_sms_clients_;
+  std::vector<int> num_kernels_;
+  std::vector<int> max_iters_;
+  std::vector<bool> is_train_;
+  int max_sms_;
+  std::vector<int> cu_masks_;
+  bool sequential_fix_;
+  // survive between schedule() calls, like the reference's globals
+  std::vector<int> seen_;
+  std::vector<int> event_ids_;
+  std::vector<int> cur_iters_;
+  std::vector<bool> stops_;
+  int penalty_ = 0;
+  // per-call state mirrored out for inspection
+  int sm_threshold_ = 0;
+  bool large_found_ = false;
+  long sum_ = 0;
+  int algo_ = ALGO_ORION;
+  bool changed_ = false;
+};
+
+}  // namespace orion
