@@ -1,0 +1,94 @@
+/* C ABI of scheduler_eval.so and of the control calls of libinttemp.so: the
+ * drop-in boundary of the scheduling hot path.  Names, argument order and
+ * meaning are those the reference's Python frontend binds through ctypes
+ * (src/scheduler_frontend.py:13,60,72,78,85,91) and its client loops call
+ * (benchmarking/benchmark_suite/train_imagenet.py:63-68,88).
+ *
+ * The reference passes Python bools as C ints and reads pointer results as
+ * 32-bit ints (ctypes defaults); both work here because every bool parameter
+ * is read from the low byte and the handle is never dereferenced.
+ */
+#ifndef ORION_SCHEDULER_H_
+#define ORION_SCHEDULER_H_
+
+#include <stdbool.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scheduler_eval.so ------------------------------------------------- */
+
+/* reference: sched_init, src/scheduler/scheduler_eval.cpp:491-495.
+ * Returns an opaque token; all state is process-global. */
+void* sched_init(void);
+
+/* reference: setup, scheduler_eval.cpp:542-660.  The LAST client is the
+ * high-priority one.  tids are the OS thread ids of the client threads; files
+ * are profile CSVs (Name,Profile,Memory_footprint,SM_usage,Duration) with at
+ * least num_kernels[i] rows.  Creates the streams (one spanning all CUs for
+ * the high-priority client, one per CU-mask size for each best-effort client)
+ * and starts routing the client threads' HIP calls through their queues.
+ * Aborts with a message on an unreadable profile (the reference asserts).
+ * Environment: ORION_BE_CU_MASKS (ascending CU counts, default
+ * cus/8,cus/4,cus/2,cus), ORION_MAX_SMS (default: the device's CU count; the
+ * reference hard-codes 80, scheduler_eval.cpp:20), ORION_RECORD_DIR (write
+ * observations.log / decisions.log there), ORION_QUIET,
+ * ORION_SEQUENTIAL_AS_WRITTEN. */
+void setup(void* scheduler, int num_clients, int* tids, char** models,
+           char** files, int* num_kernels, int* num_iters, bool* train,
+           bool reef);
+
+/* reference: setup_change, scheduler_eval.cpp:528-540: swap a client's profile
+ * and kernel count (training clients after their first iteration). */
+void setup_change(void* scheduler, int client_id, char* file, int num_kernels);
+
+/* reference: schedule, scheduler_eval.cpp:663-670 -> busy_wait_profile
+ * :238-487.  Blocks until every client has reached warmup_iters (warm-up) or
+ * its iteration limit / has acknowledged a stop (measured run).  reef / seq
+ * select the alternative policies; reef_depth is REEF's queue depth or, for
+ * the Orion policy, the budget in ns of outstanding best-effort work.
+ * Returns NULL.  After a call with warmup == false the client threads' HIP
+ * calls pass straight through again. */
+void* schedule(void* scheduler, int num_clients, bool profile_mode, int iter,
+               bool warmup, int warmup_iters, bool reef, bool seq,
+               int reef_depth, int hp_limit, int update_start);
+
+/* reference: reset, scheduler_eval.cpp:672-675. */
+void* reset(void* scheduler, int num_clients);
+
+/* No reference counterpart: stream the scheduler created for a client (its
+ * widest one), CU count in use, per-iteration wall times (ms) the scheduler
+ * measured for a client (returns how many exist, copies at most cap), and
+ * teardown of all scheduler state. */
+void* orion_client_stream(int client);
+int orion_sched_num_cus(void);
+int orion_sched_iteration_ms(int client, float* out, int cap);
+void orion_sched_teardown(void);
+
+/* ---- libinttemp.so (LD_PRELOAD) ---------------------------------------- */
+
+/* reference: block, src/cuda_capture/intercept_temp.cpp:124-130.  Called by a
+ * client thread after submitting iteration `it`; returns when the scheduler
+ * has seen all its kernels complete. */
+void block(int it);
+
+/* reference: stop, intercept_temp.cpp:132-141.  Non-zero once the scheduler
+ * asked the calling client to stop (the high-priority client is done); the
+ * call acknowledges it.  Returns int (the reference returns a C bool that its
+ * caller reads as an int). */
+int stop(void);
+
+/* No reference counterpart (the reference patches PyTorch instead,
+ * setup/orion-torch-changes.patch:779-803): tie the calling thread, or a
+ * stream the calling client thread uses, to a client, so that work issued on
+ * the client's behalf by other threads is routed to its queue. */
+void orion_register_thread(int client);
+void orion_register_stream(void* stream);
+int orion_client_index(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ORION_SCHEDULER_H_ */

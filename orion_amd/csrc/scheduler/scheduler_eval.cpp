@@ -1,0 +1,479 @@
+// scheduler_eval.so: the scheduler behind the reference's C ABI
+// (sched_init / setup / setup_change / schedule / reset,
+// src/scheduler/scheduler_eval.cpp:489-676), rebuilt for MI355X.
+//
+// The poll loop itself is the pure policy core (policy/policy.cpp).  This file
+// is its live PolicyHost: it peeks the hand-off queues of libinttemp.so, issues
+// records on HIP streams, answers completion queries with HIP events, releases
+// iterations and raises stops.
+//
+// MI355X specifics:
+//  * the high-priority client owns one stream spanning all compute units; every
+//    best-effort client owns one stream per CU-mask size
+//    (hipExtStreamCreateWithCUMask; mask bit i lands on XCD i % 8, so a run of
+//    low bits spreads evenly over the eight XCDs), and a best-effort kernel goes
+//    to the smallest mask that holds its profiled CU need;
+//  * all streams keep the default priority: streams of different priorities
+//    are not used on this platform (the reference gives the high-priority
+//    client cudaStreamCreateWithPriority(..., hp), utils_sched.cpp:119-147);
+//  * when consecutive records of a client land on different streams an event
+//    edge keeps them in program order;
+//  * completion events are recorded when the policy first asks about them, not
+//    after every record (the reference records one per dispatch,
+//    utils_sched.cpp:520, out of a pool of 30000 per client, :149-157);
+//  * calls that can block the host (allocation, free, synchronous copies and
+//    fills) are granted back to the calling thread instead of being run on the
+//    scheduler thread (the reference runs them inline, utils_sched.cpp:251-283).
+#include <dlfcn.h>
+#include <immintrin.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../capture/capture.h"
+#include "../policy/obslog.h"
+#include "../policy/policy.h"
+#include "orion_scheduler.h"
+
+extern "C" {
+int orion_execute_record(const orion::Record* rec, hipStream_t stream);
+bool orion_record_runs_on_caller(int type);
+}
+
+namespace {
+
+using namespace orion;
+using Clock = std::chrono::steady_clock;
+
+constexpr int kGrantedToCaller = -1000;  // keep equal to capture.cpp
+
+[[noreturn]] void die(const std::string& what) {
+  fprintf(stderr, "orion scheduler: %s\n", what.c_str());
+  abort();
+}
+
+void check(hipError_t err, const char* what) {
+  if (err != hipSuccess) {
+    const HipApi* hip = orion_hip_api();
+    die(std::string(what) + ": " +
+        (hip->hipGetErrorString ? hip->hipGetErrorString(err) : "HIP error"));
+  }
+}
+
+std::vector<int> parse_int_list(const char* text) {
+  std::vector<int> out;
+  if (!text) return out;
+  const char* p = text;
+  while (*p) {
+    char* end = nullptr;
+    long v = strtol(p, &end, 10);
+    if (end == p) break;
+    out.push_back((int)v);
+    p = end;
+    while (*p == ',' || *p == ' ') ++p;
+  }
+  return out;
+}
+
+class LiveHost : public PolicyHost {
+ public:
+  LiveHost(int n, int total_cus, const std::vector<int>& masks)
+      : n_(n), total_cus_(total_cus), masks_(masks) {
+    hip_ = orion_hip_api();
+    cap_ = orion_capture_state();
+    streams_.resize((size_t)n);
+    last_event_.assign((size_t)n, nullptr);
+    chain_event_.assign((size_t)n, nullptr);
+    last_recorded_.assign((size_t)n, true);
+    last_slot_.assign((size_t)n, -1);
+    last_kernel_stream_.assign((size_t)n, nullptr);
+    client_stream_.assign((size_t)n, nullptr);
+    cur_cu_slot_.assign((size_t)n, -1);
+    start_pending_.assign((size_t)n, true);
+    iter_start_.assign((size_t)n, Clock::now());
+    first_start_.assign((size_t)n, Clock::time_point());
+    dispatched_.assign((size_t)n, 0);
+    durations_ms_.resize((size_t)n);
+    create_streams();
+  }
+
+  ~LiveHost() override {
+    for (auto& set : streams_)
+      for (hipStream_t s : set)
+        if (s) (void)hip_->hipStreamDestroy(s);
+    for (hipEvent_t e : last_event_) if (e) (void)hip_->hipEventDestroy(e);
+    for (hipEvent_t e : chain_event_) if (e) (void)hip_->hipEventDestroy(e);
+    if (update_event_) (void)hip_->hipEventDestroy(update_event_);
+  }
+
+  hipStream_t home_stream(int client) const {
+    return streams_[(size_t)client].back();
+  }
+  void set_update_slot(int owner, int slot) {
+    update_owner_ = owner;
+    update_slot_ = slot;
+    update_valid_ = false;
+  }
+  void begin_phase() {
+    for (int i = 0; i < n_; ++i) first_start_[(size_t)i] = Clock::time_point();
+    phase_start_ = Clock::now();
+  }
+  const std::vector<std::vector<float>>& durations() const { return durations_ms_; }
+  double seconds_since_first(int client) const {
+    if (first_start_[(size_t)client] == Clock::time_point()) return 0.0;
+    return std::chrono::duration<double>(Clock::now() - first_start_[(size_t)client]).count();
+  }
+  double seconds_in_phase() const {
+    return std::chrono::duration<double>(Clock::now() - phase_start_).count();
+  }
+  uint64_t dispatched(int client) const { return dispatched_[(size_t)client]; }
+  uint64_t stream_switches() const { return stream_switches_; }
+
+  // ---- PolicyHost
+  void begin_poll() override { _mm_pause(); }
+
+  bool stop_ack(int client) override {
+    return cap_->channels[client].stop_ack.load(std::memory_order_acquire) != 0;
+  }
+
+  int peek(int client) override {
+    ClientChannel& ch = cap_->channels[client];
+    const uint64_t head = ch.head.load(std::memory_order_relaxed);
+    if (ch.tail.load(std::memory_order_acquire) == head) return REC_NONE;
+    if (start_pending_[(size_t)client]) {
+      // reference: client_starts[i], scheduler_eval.cpp:290-296
+      iter_start_[(size_t)client] = Clock::now();
+      start_pending_[(size_t)client] = false;
+      if (first_start_[(size_t)client] == Clock::time_point())
+        first_start_[(size_t)client] = iter_start_[(size_t)client];
+    }
+    return rec_class_of(ch.slots[head & (kQueueSlots - 1)].type);
+  }
+
+  bool event_done(int owner, int index) override {
+    if (index == last_slot_[(size_t)owner]) {
+      if (!last_recorded_[(size_t)owner]) {
+        check(hip_->hipEventRecord(last_event_[(size_t)owner],
+                                   last_kernel_stream_[(size_t)owner]),
+              "hipEventRecord");
+        last_recorded_[(size_t)owner] = true;
+      }
+      return hip_->hipEventQuery(last_event_[(size_t)owner]) == hipSuccess;
+    }
+    if (owner == update_owner_ && index == update_slot_ && update_valid_)
+      return hip_->hipEventQuery(update_event_) == hipSuccess;
+    // An index the policy can only reach after the op completed long ago.
+    return true;
+  }
+
+  int64_t iteration_us(int client) override {
+    return std::chrono::duration_cast<std::chrono::microseconds>(
+               Clock::now() - iter_start_[(size_t)client]).count();
+  }
+
+  void dispatch(const Dispatch& d) override {
+    ClientChannel& ch = cap_->channels[d.client];
+    const uint64_t head = ch.head.load(std::memory_order_relaxed);
+    Record* rec = &ch.slots[head & (kQueueSlots - 1)];
+
+    // Stream: the owner's stream set, at the slot the policy placed the kernel
+    // in; records that are not kernels stay where the client's work is.
+    auto& set = streams_[(size_t)d.owner];
+    int slot = d.cu_slot;
+    if (slot < 0) slot = cur_cu_slot_[(size_t)d.client];
+    if (slot < 0 || slot >= (int)set.size()) slot = (int)set.size() - 1;
+    hipStream_t stream = set[(size_t)slot];
+
+    hipStream_t prev = client_stream_[(size_t)d.client];
+    if (prev != nullptr && prev != stream) {
+      // keep the client's records in program order across streams
+      hipEvent_t e = chain_event_[(size_t)d.client];
+      check(hip_->hipEventRecord(e, prev), "hipEventRecord(chain)");
+      check(hip_->hipStreamWaitEvent(stream, e, 0), "hipStreamWaitEvent(chain)");
+      ++stream_switches_;
+    }
+    client_stream_[(size_t)d.client] = stream;
+    cur_cu_slot_[(size_t)d.client] = slot;
+    ch.last_stream.store(stream, std::memory_order_release);
+
+    if (orion_record_runs_on_caller(rec->type)) {
+      rec->sync_stream = stream;
+      rec->status = kGrantedToCaller;
+    } else {
+      rec->status = orion_execute_record(rec, stream);
+    }
+    if (d.rec_class == REC_KERNEL) {
+      last_kernel_stream_[(size_t)d.owner] = stream;
+      last_slot_[(size_t)d.owner] = d.event_slot;
+      last_recorded_[(size_t)d.owner] = false;
+      if (d.owner == update_owner_ && d.event_slot == update_slot_) {
+        check(hip_->hipEventRecord(update_event_, stream), "hipEventRecord(update)");
+        update_valid_ = true;
+      }
+    }
+    ++dispatched_[(size_t)d.client];
+    // pop_from_queue: retiring the record releases the caller
+    ch.head.store(head + 1, std::memory_order_release);
+  }
+
+  void iteration_done(int client, int iteration) override {
+    ClientChannel& ch = cap_->channels[client];
+    ch.released_iters.store((int64_t)iteration + 1, std::memory_order_release);
+    const float ms = (float)iteration_us(client) / 1000.0f;
+    durations_ms_[(size_t)client].push_back(ms);
+    start_pending_[(size_t)client] = true;
+    if (client == update_owner_) update_valid_ = false;
+  }
+
+  void set_stop(int client) override {
+    cap_->channels[client].stop.store(1, std::memory_order_release);
+  }
+
+ private:
+  void create_streams() {
+    for (int c = 0; c < n_; ++c) {
+      const bool is_hp = c == n_ - 1;
+      check(hip_->hipEventCreateWithFlags(&last_event_[(size_t)c], hipEventDisableTiming),
+            "hipEventCreateWithFlags");
+      check(hip_->hipEventCreateWithFlags(&chain_event_[(size_t)c], hipEventDisableTiming),
+            "hipEventCreateWithFlags");
+      if (is_hp) {
+        hipStream_t s = nullptr;
+        check(hip_->hipStreamCreateWithFlags(&s, hipStreamNonBlocking),
+              "hipStreamCreateWithFlags");
+        streams_[(size_t)c].push_back(s);
+        continue;
+      }
+      for (int m : masks_) {
+        hipStream_t s = nullptr;
+        if (m >= total_cus_ || !hip_->hipExtStreamCreateWithCUMask) {
+          check(hip_->hipStreamCreateWithFlags(&s, hipStreamNonBlocking),
+                "hipStreamCreateWithFlags");
+        } else {
+          // low m bits: m / 8 compute units on each of the eight XCDs
+          std::vector<uint32_t> words((size_t)(total_cus_ + 31) / 32, 0u);
+          for (int b = 0; b < m; ++b) words[(size_t)b / 32] |= 1u << (b % 32);
+          check(hip_->hipExtStreamCreateWithCUMask(&s, (uint32_t)words.size(), words.data()),
+                "hipExtStreamCreateWithCUMask");
+        }
+        streams_[(size_t)c].push_back(s);
+      }
+    }
+    check(hip_->hipEventCreateWithFlags(&update_event_, hipEventDisableTiming),
+          "hipEventCreateWithFlags");
+  }
+
+  int n_, total_cus_;
+  std::vector<int> masks_;
+  const HipApi* hip_;
+  CaptureState* cap_;
+  std::vector<std::vector<hipStream_t>> streams_;   // [client][cu slot]
+  std::vector<hipEvent_t> last_event_, chain_event_;
+  std::vector<char> last_recorded_;
+  std::vector<int> last_slot_;
+  std::vector<hipStream_t> last_kernel_stream_, client_stream_;
+  std::vector<int> cur_cu_slot_;
+  hipEvent_t update_event_ = nullptr;
+  int update_owner_ = -1, update_slot_ = -1;
+  bool update_valid_ = false;
+  std::vector<char> start_pending_;
+  std::vector<Clock::time_point> iter_start_, first_start_;
+  Clock::time_point phase_start_;
+  std::vector<uint64_t> dispatched_;
+  uint64_t stream_switches_ = 0;
+  std::vector<std::vector<float>> durations_ms_;
+};
+
+// All scheduler state is process-global: the reference's handle is an empty
+// object whose pointer its ctypes caller truncates to 32 bits
+// (scheduler_eval.cpp:6-46, scheduler_frontend.py:13), so the handle argument
+// of every entry point is ignored here as well.
+struct Global {
+  std::unique_ptr<Policy> policy;
+  std::unique_ptr<LiveHost> host;
+  std::unique_ptr<Recorder> recorder;
+  int n = 0;
+  int total_cus = 0;
+  std::vector<int> masks;
+  std::vector<bool> is_train;
+  std::string record_dir;
+  bool verbose = true;
+};
+Global g;
+int g_handle_token = 0;
+
+void flush_recording() {
+  if (!g.recorder || g.record_dir.empty()) return;
+  const std::string obs = g.record_dir + "/observations.log";
+  const std::string dec = g.record_dir + "/decisions.log";
+  FILE* f = fopen(obs.c_str(), "a");
+  if (f) { fwrite(g.recorder->observations().data(), 1, g.recorder->observations().size(), f); fclose(f); }
+  f = fopen(dec.c_str(), "a");
+  if (f) { fwrite(g.recorder->decisions().data(), 1, g.recorder->decisions().size(), f); fclose(f); }
+  g.recorder->clear();
+}
+
+}  // namespace
+
+extern "C" {
+
+void* sched_init(void) { return &g_handle_token; }
+
+void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
+           char** files, int* num_kernels, int* num_iters, bool* train, bool /*reef*/) {
+  if (num_clients < 1 || num_clients > kMaxClients) die("client count out of range");
+  const HipApi* hip = orion_hip_api();
+  const pid_t mytid = (pid_t)syscall(SYS_gettid);
+
+  int cus = 0;
+  if (const char* e = getenv("ORION_MAX_SMS")) cus = atoi(e);
+  if (cus <= 0) {
+    int dev = 0;
+    if (hip->hipGetDevice) (void)hip->hipGetDevice(&dev);
+    check(hip->hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
+          "hipDeviceGetAttribute(MultiprocessorCount)");
+  }
+  g.total_cus = cus;
+  g.masks = parse_int_list(getenv("ORION_BE_CU_MASKS"));
+  if (g.masks.empty()) g.masks = {cus / 8, cus / 4, cus / 2, cus};
+  for (size_t i = 0; i < g.masks.size(); ++i)
+    if (g.masks[i] <= 0 || (i && g.masks[i] <= g.masks[i - 1]))
+      die("ORION_BE_CU_MASKS must be an ascending list of positive CU counts");
+  if (g.masks.back() < cus) g.masks.push_back(cus);
+  if (const char* e = getenv("ORION_QUIET")) g.verbose = atoi(e) == 0;
+
+  std::vector<std::vector<OpInfo>> profiles((size_t)num_clients);
+  std::vector<int> nk, ni;
+  g.is_train.clear();
+  for (int i = 0; i < num_clients; ++i) {
+    std::string err;
+    if (!parse_profile(files[i], &profiles[(size_t)i], &err)) die(err);
+    if ((int)profiles[(size_t)i].size() < num_kernels[i])
+      die(std::string(files[i]) + ": fewer rows than num_kernels");
+    if (g.verbose)
+      printf("KERNEL_INFO_FILE IS %s\n----------- SIZE: %zu\n", files[i],
+             profiles[(size_t)i].size());
+    nk.push_back(num_kernels[i]);
+    ni.push_back(num_iters[i]);
+    g.is_train.push_back(train[i]);
+  }
+  const bool as_written = getenv("ORION_SEQUENTIAL_AS_WRITTEN") &&
+                          atoi(getenv("ORION_SEQUENTIAL_AS_WRITTEN")) != 0;
+  g.n = num_clients;
+  g.host.reset();  // streams of a previous job first
+  g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, cus, g.masks,
+                            !as_written));
+  g.host.reset(new LiveHost(num_clients, cus, g.masks));
+  g.recorder.reset();
+  g.record_dir.clear();
+  if (const char* dir = getenv("ORION_RECORD_DIR")) {
+    if (*dir) {
+      g.record_dir = dir;
+      g.recorder.reset(new Recorder(g.host.get(), num_clients));
+      g.recorder->header(cus, g.masks);
+      for (int i = 0; i < num_clients; ++i)
+        g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
+      // start both logs afresh
+      FILE* f = fopen((g.record_dir + "/observations.log").c_str(), "w");
+      if (f) fclose(f);
+      f = fopen((g.record_dir + "/decisions.log").c_str(), "w");
+      if (f) fclose(f);
+    }
+  }
+  orion_capture_arm(num_clients, tids, (int)mytid);
+}
+
+void setup_change(void* /*scheduler*/, int client_id, char* file, int num_kernels) {
+  if (!g.policy || client_id < 0 || client_id >= g.n) die("setup_change before setup");
+  std::vector<OpInfo> ops;
+  std::string err;
+  if (!parse_profile(file, &ops, &err)) die(err);
+  if ((int)ops.size() < num_kernels) die(std::string(file) + ": fewer rows than num_kernels");
+  if (g.verbose) printf("KERNEL_INFO_FILE IS %s\n", file);
+  g.policy->setup_change(client_id, std::move(ops), num_kernels);
+  if (g.recorder) g.recorder->setup_change(client_id, num_kernels, file);
+}
+
+void* schedule(void* /*scheduler*/, int num_clients, bool profile_mode, int /*iter*/,
+               bool warmup, int warmup_iters, bool reef, bool seq, int reef_depth,
+               int hp_limit, int update_start) {
+  if (!profile_mode) return nullptr;  // scheduler_eval.cpp:666
+  if (!g.policy || num_clients != g.n) die("schedule before setup");
+  ScheduleArgs a;
+  a.warmup = warmup;
+  a.warmup_iters = warmup_iters;
+  a.algo = reef ? ALGO_REEF : (seq ? ALGO_SEQUENTIAL : ALGO_ORION);
+  a.depth = reef_depth;
+  a.hp_limit = hp_limit;
+  a.update_start = update_start;
+  const int hp = g.n - 1;
+  if (g.is_train[(size_t)hp] && a.algo == ALGO_ORION)
+    g.host->set_update_slot(hp, update_start - 1);
+  else
+    g.host->set_update_slot(-1, -1);
+  g.host->begin_phase();
+  PolicyHost* host = g.host.get();
+  if (g.recorder) {
+    g.recorder->set_inner(g.host.get());
+    g.recorder->begin_schedule(a);
+    host = g.recorder.get();
+  }
+  g.policy->schedule(*host, a);
+  if (g.recorder) {
+    g.recorder->end_schedule();
+    flush_recording();
+  }
+  if (!warmup) {
+    // scheduler_eval.cpp:455-462, :478-482
+    if (g.verbose) {
+      for (int i = 0; i < g.n; ++i)
+        printf("Client %d, Total loop took %f sec, %d iterations, %llu records\n", i,
+               g.host->seconds_since_first(i), g.policy->cur_iters()[(size_t)i],
+               (unsigned long long)g.host->dispatched(i));
+      printf("Total loop took %f sec (%llu cross-stream edges)\n",
+             g.host->seconds_in_phase(), (unsigned long long)g.host->stream_switches());
+      fflush(stdout);
+    }
+    // The measured run is over: whatever clients issue from now on is theirs.
+    orion_capture_disarm();
+  }
+  return nullptr;
+}
+
+void* reset(void* /*scheduler*/, int /*num_clients*/) {
+  // profile_reset (scheduler_eval.cpp:49-56) only clears per-iteration
+  // counters that the policy core clears itself when an iteration completes.
+  return nullptr;
+}
+
+void* orion_client_stream(int client) {
+  if (!g.host || client < 0 || client >= g.n) return nullptr;
+  return (void*)g.host->home_stream(client);
+}
+
+int orion_sched_num_cus(void) { return g.total_cus; }
+
+int orion_sched_iteration_ms(int client, float* out, int cap) {
+  if (!g.host || client < 0 || client >= g.n) return -1;
+  const auto& d = g.host->durations()[(size_t)client];
+  int k = (int)d.size() < cap ? (int)d.size() : cap;
+  for (int i = 0; i < k; ++i) out[i] = d[(size_t)i];
+  return (int)d.size();
+}
+
+void orion_sched_teardown(void) {
+  orion_capture_disarm();
+  g.recorder.reset();
+  g.host.reset();
+  g.policy.reset();
+  g.n = 0;
+}
+
+}  // extern "C"

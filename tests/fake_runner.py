@@ -1,0 +1,165 @@
+"""Drives libinttemp.so + scheduler_eval.so end to end on a host without a GPU,
+against the recording HIP stand-in (tests/fakehip).  Runs in its own process
+(the HIP table of a process is resolved once); prints one JSON object.
+
+usage: python tests/fake_runner.py <workdir> <algo> <n_be> <hp_iters>
+"""
+
+import ctypes
+import json
+import os
+import sys
+import threading
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+os.environ["ORION_HIP_LIBRARY"] = os.path.join(ROOT, "tests", "fakehip", "libfakehip.so")
+
+import numpy as np  # noqa: E402
+
+from orion_amd import _lib, scheduler_frontend as fe  # noqa: E402
+
+workdir, algo, n_be, hp_iters = sys.argv[1], sys.argv[2], int(sys.argv[3]), int(sys.argv[4])
+os.environ["ORION_RECORD_DIR"] = workdir
+os.environ["ORION_QUIET"] = "1"
+
+fake = ctypes.CDLL(os.environ["ORION_HIP_LIBRARY"])
+cap = fe.load_capture_library()
+sched = fe.load_scheduler_library()
+fake.fakehip_set_costs(ctypes.c_longlong(30000), ctypes.c_longlong(4000))
+
+SAXPY = ctypes.cast(fake.fake_kernel_saxpy, ctypes.c_void_p)
+SQADD = ctypes.cast(fake.fake_kernel_sqadd, ctypes.c_void_p)
+cap.hipModuleLaunchKernel.argtypes = [ctypes.c_void_p] + [ctypes.c_uint] * 7 + [
+    ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p]
+cap.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                               ctypes.c_int, ctypes.c_void_p]
+cap.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+cap.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+cap.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+
+N = 64
+n_clients = n_be + 1
+kernels_per_iter = [5 + c for c in range(n_clients)]
+iters = [10_000] * n_be + [hp_iters]
+
+
+def write_profile(path, nk, seed):
+    rng = np.random.default_rng(seed)
+    with open(path, "w") as f:
+        f.write("Name,Profile,Memory_footprint,SM_usage,Duration\n")
+        for i in range(nk):
+            f.write(f"k{i},{int(rng.integers(-1, 2))},0,{int(rng.integers(1, 300))},"
+                    f"{int(rng.integers(5000, 60000))}\n")
+
+
+files = []
+for c in range(n_clients):
+    p = os.path.join(workdir, f"client{c}.csv")
+    write_profile(p, kernels_per_iter[c], c)
+    files.append(p)
+
+results = [None] * n_clients
+iters_done = [0] * n_clients
+barriers = [threading.Barrier(n_clients + 1)]
+
+
+def launch(func, params):
+    arr = (ctypes.c_void_p * len(params))(*[ctypes.cast(ctypes.pointer(p), ctypes.c_void_p)
+                                            for p in params])
+    rc = cap.hipModuleLaunchKernel(func, 1, 1, 1, 64, 1, 1, 0, None, arr, None)
+    assert rc == 0, rc
+
+
+def client(tid):
+    nk = kernels_per_iter[tid]
+    host_x = np.arange(N, dtype=np.float32) / N + tid
+    barriers[0].wait()
+    dev_y, dev_x = ctypes.c_void_p(), ctypes.c_void_p()
+    assert cap.hipMalloc(ctypes.byref(dev_y), N * 4) == 0
+    assert cap.hipMalloc(ctypes.byref(dev_x), N * 4) == 0
+    zeros = np.zeros(N, dtype=np.float32)
+    cap.hipMemcpy(dev_y, zeros.ctypes.data, N * 4, 1)
+    it = 0
+    n_c, a_c = ctypes.c_int(N), ctypes.c_float(0.5)
+    c_c = ctypes.c_float(0.125)
+    while it < iters[tid]:
+        cap.hipMemcpyAsync(dev_x, host_x.ctypes.data, N * 4, 1, None)
+        for k in range(nk):
+            if k % 2 == 0:
+                launch(SAXPY, [dev_y, dev_x, a_c, n_c])
+            else:
+                launch(SQADD, [dev_y, c_c, n_c])
+        cap.block(it)
+        it += 1
+        iters_done[tid] = it
+        if it in (1, 10):
+            barriers[0].wait()
+        if cap.stop():
+            break
+    barriers[0].wait()
+    out = np.empty(N, dtype=np.float32)
+    cap.hipMemcpy(out.ctypes.data, dev_y, N * 4, 2)
+    results[tid] = out
+
+
+def expected(tid, n_iters):
+    nk = kernels_per_iter[tid]
+    x = np.arange(N, dtype=np.float32) / N + tid
+    y = np.zeros(N, dtype=np.float32)
+    with np.errstate(over="ignore"):
+        for _ in range(n_iters):
+            for k in range(nk):
+                if k % 2 == 0:
+                    y = np.float32(0.5) * x + y
+                else:
+                    y = y * y + np.float32(0.125)
+    return y
+
+
+threads = [threading.Thread(target=client, args=(c,)) for c in range(n_clients)]
+for t in threads:
+    t.start()
+tids = [t.native_id for t in threads]
+py = fe.PyScheduler(sched, n_clients)
+sched_tid = []
+
+
+def run_sched():
+    sched_tid.append(threading.get_native_id())
+    py.run_scheduler(barriers, tids, ["fake"] * n_clients, files,
+                     [None] * n_clients, kernels_per_iter, [None] * n_clients,
+                     iters, True, True, algo == "reef", algo == "sequential",
+                     8 if algo == "reef" else 100_000, 1, 1, [True] * n_be + [False])
+
+
+st = threading.Thread(target=run_sched)
+st.start()
+for t in threads:
+    t.join(timeout=120)
+st.join(timeout=120)
+alive = [t.is_alive() for t in threads] + [st.is_alive()]
+
+log = []
+kind, sid, tid_, a, b = (ctypes.c_int(), ctypes.c_int(), ctypes.c_int(),
+                         ctypes.c_ulonglong(), ctypes.c_ulonglong())
+for i in range(fake.fakehip_log_size()):
+    fake.fakehip_log_get(i, ctypes.byref(kind), ctypes.byref(sid), ctypes.byref(tid_),
+                         ctypes.byref(a), ctypes.byref(b))
+    log.append((kind.value, sid.value, tid_.value))
+launch_tids = sorted({t for k, s, t in log if k == 0})
+launch_streams = sorted({s for k, s, t in log if k == 0})
+masks = {s: fake.fakehip_stream_mask_bits(s) for s in launch_streams}
+
+ok_outputs = []
+for c in range(n_clients):
+    want = expected(c, iters_done[c])
+    ok_outputs.append(bool(results[c] is not None and np.array_equal(results[c], want)))
+
+print(json.dumps({
+    "alive": alive, "iters_done": iters_done, "outputs_equal": ok_outputs,
+    "launch_tids": launch_tids, "sched_tid": sched_tid, "client_tids": tids,
+    "launch_stream_masks": masks, "n_launches": sum(1 for k, s, t in log if k == 0),
+}))
+sys.stdout.flush()
+os._exit(0 if not any(alive) else 3)
