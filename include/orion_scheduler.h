@@ -67,6 +67,18 @@ int orion_sched_num_cus(void);
 int orion_sched_iteration_ms(int client, float* out, int cap);
 void orion_sched_teardown(void);
 
+/* Profile capture (no reference counterpart; replaces the Nsight runs of
+ * PROFILE.md:7-54).  orion_profile_begin routes the client thread `client_tid`
+ * through the interception layer and opens the trace file; orion_profile_run
+ * serves it alone, in order, timing every kernel with HIP events, until it has
+ * completed `until_iteration` iterations (an iteration ends at block());
+ * orion_profile_end stops routing and closes the trace.  Trace columns:
+ * iteration,index,type,name,grid_x..z,block_x..z,dyn_lds,regs,static_lds,
+ * duration_ns.  All return 0 on success. */
+int orion_profile_begin(int client_tid, const char* trace_path);
+int orion_profile_run(int until_iteration);
+int orion_profile_end(void);
+
 /* ---- libinttemp.so (LD_PRELOAD) ---------------------------------------- */
 
 /* reference: block, src/cuda_capture/intercept_temp.cpp:124-130.  Called by a
@@ -87,6 +99,12 @@ int stop(void);
 void orion_register_thread(int client);
 void orion_register_stream(void* stream);
 int orion_client_index(void);
+
+/* No reference counterpart: while on, the calling thread's HIP calls bypass the
+ * queues.  Client loops use it around model construction and library
+ * auto-tuning, whose kernel count differs from run to run on ROCm and would
+ * otherwise never match a profile's row count. */
+void orion_thread_passthrough(int on);
 
 #ifdef __cplusplus
 }

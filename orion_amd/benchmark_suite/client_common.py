@@ -1,0 +1,167 @@
+"""What every client loop shares: the control calls into libinttemp.so, the
+arrival schedule, the request loop with its barrier protocol, and the result
+file.  Behaviour follows the reference's loops
+(benchmarking/benchmark_suite/train_imagenet.py:71-241,
+bert_trainer_mock.py:49-234); the line numbers below are train_imagenet.py's.
+"""
+
+import json
+import os
+import random
+import time
+
+import numpy as np
+import torch
+
+from .. import scheduler_frontend as fe
+
+WARMUP_ITERS = 10     # iterations before the measured run (:188-198, :220)
+
+
+def seed_everything(seed):
+    """:22-30."""
+    random.seed(seed)
+    os.environ["PYTHONHASHSEED"] = str(seed)
+    np.random.seed(seed)
+    torch.manual_seed(seed)
+    if torch.cuda.is_available():
+        torch.cuda.manual_seed(seed)
+
+
+def arrival_gaps(rps, uniform, num_iters, input_file="", seed=42):
+    """Inter-arrival gaps in seconds (:89-98): constant 1/rps, exponential with
+    mean 1/rps from a generator seeded like the reference's global numpy seed,
+    a JSON trace, or zeros (closed loop)."""
+    if rps > 0 and input_file == "":
+        if uniform:
+            return [1.0 / rps] * num_iters
+        return list(np.random.RandomState(seed).exponential(scale=1.0 / rps,
+                                                            size=num_iters))
+    if input_file != "":
+        with open(input_file) as f:
+            return list(json.load(f))
+    return [0.0] * num_iters
+
+
+def latency_summary(timings, batch_idx, total_time, train, drop=WARMUP_ITERS):
+    """Result dictionary of a client (:220-237): drop the warm-up requests,
+    percentiles in milliseconds, throughput over the measured run."""
+    timings = sorted(timings[drop:])
+    throughput = (batch_idx - WARMUP_ITERS) / total_time if total_time > 0 else 0.0
+    if not train and len(timings) > 0:
+        return {
+            "p50_latency": float(np.percentile(timings, 50) * 1000),
+            "p95_latency": float(np.percentile(timings, 95) * 1000),
+            "p99_latency": float(np.percentile(timings, 99) * 1000),
+            "throughput": throughput,
+        }
+    return {"throughput": throughput}
+
+
+def write_result(tid, data):
+    out_dir = os.environ.get("ORION_RESULT_DIR", ".")
+    with open(os.path.join(out_dir, f"client_{tid}.json"), "w") as f:
+        json.dump(data, f)
+
+
+class Backend:
+    """block()/stop() of libinttemp.so (:63-68, :88) plus stream registration."""
+
+    def __init__(self):
+        self.lib = fe.load_capture_library()
+
+    def block(self, it):
+        self.lib.block(it)
+
+    def stop(self):
+        return bool(self.lib.stop())
+
+    def register_stream(self, stream):
+        self.lib.orion_register_stream(stream.cuda_stream)
+
+    def passthrough(self, on):
+        self.lib.orion_thread_passthrough(1 if on else 0)
+
+
+class uncaptured:
+    """Context in which the calling thread's GPU work bypasses the scheduler.
+
+    On ROCm the first executions of a model run library auto-tuning (MIOpen
+    tries several convolution solvers and times them) and lazy initialisation
+    whose number of kernels is not reproducible, so no profile could name a row
+    count for them.  A client therefore builds its model and runs its first
+    steps here, synchronises, and only then starts the iterations the scheduler
+    counts."""
+
+    def __init__(self, backend):
+        self.backend = backend
+
+    def __enter__(self):
+        self.backend.passthrough(True)
+
+    def __exit__(self, *exc):
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+        self.backend.passthrough(False)
+        return False
+
+UNCAPTURED_STEPS = 3  # auto-tuning, lazy init, first optimizer step, one more
+
+
+def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
+               drop=WARMUP_ITERS, extra=None):
+    """The request loop.  ``step(batch_idx)`` submits one iteration's GPU work.
+
+    Training clients run closed loop (:141-169).  Inference clients run open
+    loop (:170-204): request i is due at ``next_startup``; its latency counts
+    from that due time, so queueing delay is included; the due time advances by
+    the arrival gap once the client is past warm-up.  Both rendezvous with the
+    scheduler on ``barriers[0]`` after iterations 1 and 10 and once at the end.
+    """
+    timings = []
+    batch_idx = 0
+    start = time.time()
+    next_startup = time.time()
+    while batch_idx < num_iters:
+        if train:
+            start_iter = time.time()
+            step(batch_idx)
+            backend.block(batch_idx)
+            timings.append(time.time() - start_iter)
+            batch_idx += 1
+            if batch_idx == 1:
+                barriers[0].wait()
+            if batch_idx == WARMUP_ITERS:
+                barriers[0].wait()
+                start = time.time()
+            if backend.stop():
+                break
+        else:
+            if time.time() < next_startup:
+                continue
+            step(batch_idx)
+            backend.block(batch_idx)
+            timings.append(time.time() - next_startup)
+            if batch_idx >= WARMUP_ITERS:
+                next_startup += sleep_times[batch_idx]
+            else:
+                next_startup = time.time()
+            batch_idx += 1
+            if batch_idx in (1, WARMUP_ITERS):
+                barriers[0].wait()
+                if batch_idx == WARMUP_ITERS:
+                    next_startup = time.time()
+                    start = time.time()
+            dur = next_startup - time.time()
+            if dur > 0:
+                time.sleep(dur)
+            if backend.stop():
+                break
+    barriers[0].wait()
+    total_time = time.time() - start
+    data = latency_summary(timings, batch_idx, total_time, train, drop)
+    if extra:
+        data.update(extra())
+    data["iterations"] = batch_idx
+    write_result(tid, data)
+    return data

@@ -220,6 +220,7 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
     ch.stop_ack.store(0);
     ch.last_stream.store(nullptr);
     ch.submitted.store(0);
+    ch.block_calls.store(0);
     // own_streams survive: a client may register its stream before setup runs
   }
   g_state.epoch.fetch_add(1, std::memory_order_acq_rel);
@@ -261,6 +262,11 @@ void orion_register_stream(void* stream) {
 
 int orion_client_index(void) { return client_for_call(nullptr); }
 
+// While on, the calling thread's HIP calls go straight to the runtime: used by
+// a client for work that must not count as part of an iteration (building the
+// model, library auto-tuning runs whose kernel count is not reproducible).
+void orion_thread_passthrough(int on) { tl_bypass = on ? 1 : 0; }
+
 // -- control calls of the client loops (reference: intercept_temp.cpp:124-142)
 
 // Returns once the scheduler has released iteration `it` of the calling client.
@@ -268,6 +274,7 @@ void block(int it) {
   const int idx = client_for_call(nullptr);
   if (idx < 0) return;  // not armed, or not a client: nothing to wait for
   ClientChannel& ch = g_state.channels[idx];
+  ch.block_calls.store((int64_t)it + 1, std::memory_order_release);
   unsigned spins = 0;
   while (ch.released_iters.load(std::memory_order_acquire) <= (int64_t)it) {
     if (!g_state.armed.load(std::memory_order_acquire)) return;

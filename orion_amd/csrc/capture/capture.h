@@ -136,6 +136,7 @@ struct alignas(64) ClientChannel {
   // behalf by threads that are not registered (autograd workers)
   std::atomic<hipStream_t> own_streams[4];
   std::atomic<uint64_t> submitted;      // records pushed, all types
+  std::atomic<int64_t> block_calls;     // highest it+1 the client passed to block()
 };
 
 struct CaptureState {

@@ -86,6 +86,8 @@ namespace orion {
   X(hipGetDevice, hipError_t, (int*))                                                       \
   X(hipGetLastError, hipError_t, (void))                                                    \
   X(hipGetErrorString, const char*, (hipError_t))                                           \
+  X(hipFuncGetAttributes, hipError_t, (struct hipFuncAttributes*, const void*))             \
+  X(hipFuncGetAttribute, hipError_t, (int*, hipFunction_attribute, hipFunction_t))          \
   X(hipKernelNameRef, const char*, (const hipFunction_t))                                   \
   X(hipKernelNameRefByPtr, const char*, (const void*, hipStream_t))
 

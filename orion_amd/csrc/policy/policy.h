@@ -112,6 +112,7 @@ class Policy {
   int num_clients() const { return n_; }
   const std::vector<int>& cur_iters() const { return cur_iters_; }
   const std::vector<int>& seen() const { return seen_; }
+  const std::vector<int>& num_kernels() const { return num_kernels_; }
   const std::vector<OpInfo>& ops(int client) const { return ops_[client]; }
   int sm_threshold() const { return sm_threshold_; }
   bool large_found() const { return large_found_; }

@@ -136,8 +136,13 @@ class LiveHost : public PolicyHost {
   uint64_t dispatched(int client) const { return dispatched_[(size_t)client]; }
   uint64_t stream_switches() const { return stream_switches_; }
 
+  void set_policy(const Policy* p) { policy_ = p; }
+
   // ---- PolicyHost
-  void begin_poll() override { _mm_pause(); }
+  void begin_poll() override {
+    _mm_pause();
+    if ((++polls_ & 0xfffff) == 0) watchdog();
+  }
 
   bool stop_ack(int client) override {
     return cap_->channels[client].stop_ack.load(std::memory_order_acquire) != 0;
@@ -237,6 +242,39 @@ class LiveHost : public PolicyHost {
   }
 
  private:
+  // The reference spins forever when a client's kernel count disagrees with its
+  // profile (scheduler_eval.cpp:282, :389).  Here that state -- the client
+  // waits in block() with an empty queue while the policy still expects more
+  // kernels -- is reported and ends the process once it has lasted a while.
+  void watchdog() {
+    if (!policy_) return;
+    const auto now = Clock::now();
+    for (int i = 0; i < n_; ++i) {
+      ClientChannel& ch = cap_->channels[i];
+      const bool waiting = ch.block_calls.load(std::memory_order_acquire) >
+                           ch.released_iters.load(std::memory_order_acquire);
+      const bool empty = ch.tail.load(std::memory_order_acquire) ==
+                         ch.head.load(std::memory_order_acquire);
+      const int seen = policy_->seen()[(size_t)i];
+      const int want = policy_->num_kernels()[(size_t)i];
+      if (waiting && empty && seen != want && seen != 0) {
+        if (stuck_since_.size() != (size_t)n_) stuck_since_.assign((size_t)n_, Clock::time_point());
+        if (stuck_since_[(size_t)i] == Clock::time_point()) {
+          stuck_since_[(size_t)i] = now;
+        } else if (std::chrono::duration<double>(now - stuck_since_[(size_t)i]).count() > stuck_limit_s_) {
+          char msg[256];
+          snprintf(msg, sizeof msg,
+                   "client %d submitted %d kernel records in this iteration and waits in "
+                   "block(), but its profile names %d (num_kernels): the job file and the "
+                   "profile do not match this client", i, seen, want);
+          die(msg);
+        }
+      } else if (stuck_since_.size() == (size_t)n_) {
+        stuck_since_[(size_t)i] = Clock::time_point();
+      }
+    }
+  }
+
   void create_streams() {
     for (int c = 0; c < n_; ++c) {
       const bool is_hp = c == n_ - 1;
@@ -272,6 +310,10 @@ class LiveHost : public PolicyHost {
 
   int n_, total_cus_;
   std::vector<int> masks_;
+  const Policy* policy_ = nullptr;
+  uint64_t polls_ = 0;
+  std::vector<Clock::time_point> stuck_since_;
+  double stuck_limit_s_ = getenv("ORION_STUCK_LIMIT_S") ? atof(getenv("ORION_STUCK_LIMIT_S")) : 20.0;
   const HipApi* hip_;
   CaptureState* cap_;
   std::vector<std::vector<hipStream_t>> streams_;   // [client][cu slot]
@@ -371,6 +413,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
   g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, cus, g.masks,
                             !as_written));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
+  g.host->set_policy(g.policy.get());
   g.recorder.reset();
   g.record_dir.clear();
   if (const char* dir = getenv("ORION_RECORD_DIR")) {

@@ -1,0 +1,76 @@
+"""From a kernel's launch shape and resource use to the two profile columns the
+policy reads: the compute units it can occupy and its bound class.
+
+Counterpart of the reference's ``profiling/postprocessing/get_num_blocks.py``
+(``SM_needed``, :34-52) and ``roofline_analysis.py`` (class, :37-71), restated
+for a CDNA4 compute unit instead of a V100 SM:
+
+* 4 SIMDs per CU, at most 8 resident wavefronts of 64 lanes each per SIMD;
+* 512 vector registers per lane and SIMD (architectural + accumulation
+  registers are one file), allocated in blocks of 8;
+* 160 KiB of LDS per CU;
+* at most 32 resident workgroups per CU.
+"""
+
+from math import ceil
+
+WAVE = 64
+SIMDS_PER_CU = 4
+MAX_WAVES_PER_SIMD = 8
+VGPRS_PER_SIMD = 512
+VGPR_GRANULE = 8
+LDS_PER_CU = 160 * 1024
+MAX_WORKGROUPS_PER_CU = 32
+
+
+def workgroups_per_cu(threads_per_block, regs_per_thread=0, lds_per_block=0):
+    """How many workgroups of this shape fit on one CU at once."""
+    waves_per_block = max(1, ceil(threads_per_block / WAVE))
+    waves_per_simd = MAX_WAVES_PER_SIMD
+    if regs_per_thread > 0:
+        alloc = ceil(regs_per_thread / VGPR_GRANULE) * VGPR_GRANULE
+        waves_per_simd = max(1, min(MAX_WAVES_PER_SIMD, VGPRS_PER_SIMD // alloc))
+    by_waves = max(1, (SIMDS_PER_CU * waves_per_simd) // waves_per_block)
+    by_lds = by_waves
+    if lds_per_block > 0:
+        by_lds = max(1, LDS_PER_CU // lds_per_block)
+    return max(1, min(by_waves, by_lds, MAX_WORKGROUPS_PER_CU))
+
+
+def cu_needed(num_blocks, threads_per_block, regs_per_thread=0, lds_per_block=0):
+    """``SM_needed`` for CDNA4: workgroups / resident workgroups per CU, not
+    clipped to the device (the reference does not clip either)."""
+    return max(1, ceil(num_blocks / workgroups_per_cu(threads_per_block,
+                                                      regs_per_thread,
+                                                      lds_per_block)))
+
+
+COMPUTE_HINTS = ("gemm", "cijk", "conv", "igemm", "winograd", "xdlops", "mfma",
+                 "attn", "fmha", "wrw", "fwd_gtc", "bwd_gtc", "implicit",
+                 "naive_conv")
+MEMORY_HINTS = ("elementwise", "batch_norm", "batchnorm", "bn_", "reduce", "pool",
+                "copy", "fill", "softmax", "layer_norm", "layernorm", "cat",
+                "index", "embedding", "dropout", "multi_tensor", "transpose",
+                "add", "mul", "relu", "scatter", "gather", "nll", "sum", "triad")
+
+
+def classify(name, hbm_fraction=None, mfma_fraction=None, threshold=0.6):
+    """1 compute-bound, 0 memory-bound, -1 unknown.
+
+    With hardware counters (fractions of peak HBM bandwidth and of peak matrix
+    throughput, from rocprofv3) the reference's utilisation rule applies
+    (roofline_analysis.py:60-66: >= 60 % decides).  Without them the kernel
+    name decides, which is what the reference's op grouping amounts to for
+    library ops (generate_file.py:62-86 labels cuDNN/cuBLAS ops by name)."""
+    if mfma_fraction is not None and mfma_fraction >= threshold:
+        return 1
+    if hbm_fraction is not None and hbm_fraction >= threshold:
+        return 0
+    if hbm_fraction is not None and mfma_fraction is not None:
+        return -1
+    low = name.lower()
+    if any(h in low for h in COMPUTE_HINTS):
+        return 1
+    if any(h in low for h in MEMORY_HINTS):
+        return 0
+    return -1

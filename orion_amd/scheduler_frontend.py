@@ -61,6 +61,8 @@ def load_capture_library(path=None):
     lib.orion_register_stream.restype = None
     lib.orion_client_index.argtypes = []
     lib.orion_client_index.restype = c_int
+    lib.orion_thread_passthrough.argtypes = [c_int]
+    lib.orion_thread_passthrough.restype = None
     lib._orion_typed = True
     return lib
 

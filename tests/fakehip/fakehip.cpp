@@ -271,6 +271,10 @@ hipError_t hipEventSynchronize(hipEvent_t e) {
   while (now_ns() < ((FakeEvent*)e)->done_at.load()) {}
   return hipSuccess;
 }
+hipError_t hipEventElapsedTime(float* ms, hipEvent_t a, hipEvent_t b) {
+  *ms = (float)(((FakeEvent*)b)->done_at.load() - ((FakeEvent*)a)->done_at.load()) / 1.0e6f;
+  return hipSuccess;
+}
 hipError_t hipDeviceSynchronize(void) {
   std::vector<FakeStream*> all;
   { std::lock_guard<std::mutex> l(g_mu); all = g_streams; }
