@@ -42,6 +42,15 @@ int orion_triad_f32(float* a, const float* b, const float* c, float s,
 int orion_gemm_bf16_nt(const void* A, const void* B, void* C, int M, int N,
                        int K, int out_is_f32, void* stream);
 
+/* A non-blocking, default-priority stream limited to the first cu_count
+ * compute units of the CU mask (hipExtStreamCreateWithCUMask; mask bit i lands
+ * on XCD i % 8), or spanning the whole GPU when cu_count <= 0 or >= the CU
+ * count.  The reference creates its streams inside the scheduler only
+ * (src/scheduler/utils_sched.cpp:119-147); this pair exists for measuring the
+ * kernels on masked streams without the scheduler. */
+int orion_stream_create(int cu_count, void** stream_out);
+int orion_stream_destroy(void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -142,9 +142,12 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
             step(batch_idx)
             backend.block(batch_idx)
             timings.append(time.time() - next_startup)
-            if batch_idx >= WARMUP_ITERS:
+            if batch_idx >= WARMUP_ITERS and sleep_times[batch_idx] > 0:
                 next_startup += sleep_times[batch_idx]
             else:
+                # warm-up, or a closed loop (rps 0): the next request is due now.
+                # (The reference adds a zero gap here, :188-189, which leaves the
+                # due time in the past and inflates every later latency.)
                 next_startup = time.time()
             batch_idx += 1
             if batch_idx in (1, WARMUP_ITERS):

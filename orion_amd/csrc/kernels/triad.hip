@@ -93,3 +93,32 @@ extern "C" int orion_triad_f32(float* a, const float* b, const float* c,
                      n_vec4, n);
   return hipGetLastError() == hipSuccess ? ORION_OK : ORION_ERR_LAUNCH;
 }
+
+// Stream helper for callers that hold no HIP binding of their own (the Python
+// layer): a non-blocking stream spanning `cu_count` compute units (the first
+// cu_count mask bits; bit i lands on XCD i % 8), or the whole GPU when
+// cu_count <= 0 or covers every CU.  Default priority.
+extern "C" int orion_stream_create(int cu_count, void** stream_out) {
+  if (stream_out == nullptr) return ORION_ERR_ARG;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return ORION_ERR_LAUNCH;
+  hipStream_t s = nullptr;
+  hipError_t err;
+  if (cu_count <= 0 || cu_count >= cus) {
+    err = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+  } else {
+    uint32_t words[16] = {0};
+    if (cus > 512) return ORION_ERR_ARG;
+    for (int b = 0; b < cu_count; ++b) words[b / 32] |= 1u << (b % 32);
+    err = hipExtStreamCreateWithCUMask(&s, (uint32_t)((cus + 31) / 32), words);
+  }
+  if (err != hipSuccess) return ORION_ERR_LAUNCH;
+  *stream_out = (void*)s;
+  return ORION_OK;
+}
+
+extern "C" int orion_stream_destroy(void* stream) {
+  return hipStreamDestroy((hipStream_t)stream) == hipSuccess ? ORION_OK : ORION_ERR_LAUNCH;
+}

@@ -31,8 +31,22 @@ def lib():
             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
             ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         handle.orion_gemm_bf16_nt.restype = ctypes.c_int
+        handle.orion_stream_create.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+        handle.orion_stream_create.restype = ctypes.c_int
+        handle.orion_stream_destroy.argtypes = [ctypes.c_void_p]
+        handle.orion_stream_destroy.restype = ctypes.c_int
         handle._orion_typed = True
     return handle
+
+
+def cu_masked_stream(cu_count, device=0):
+    """A ``torch.cuda.ExternalStream`` over a stream limited to ``cu_count``
+    compute units (the whole GPU for ``cu_count <= 0``)."""
+    out = ctypes.c_void_p()
+    rc = lib().orion_stream_create(int(cu_count), ctypes.byref(out))
+    if rc != 0:
+        raise KernelError("orion_stream_create", rc)
+    return torch.cuda.ExternalStream(out.value, device=device)
 
 
 def _stream_ptr(stream):

@@ -25,7 +25,10 @@ def _function_dict():
     # imported lazily: the model code needs torch, the argument parser does not
     from .benchmark_suite.bert_trainer import bert_loop
     from .benchmark_suite.train_imagenet import imagenet_loop
+    from .kernel_pair import gemm_loop, triad_loop
     return {
+        "gemm_bf16": gemm_loop,
+        "triad_f32": triad_loop,
         "resnet50": imagenet_loop,
         "resnet101": imagenet_loop,
         "mobilenet_v2": imagenet_loop,
