@@ -46,26 +46,31 @@ class DecisionLog:
         return "\n".join(self.lines) + ("\n" if self.lines else "")
 
 
-def place_cu_slot(masks, cls, sm_used, algo):
+def place_cu_slot(masks, cls, sm_used, algo, hp_active):
     """CU-mask placement of a best-effort dispatch (no reference counterpart:
     the reference has one stream per client).  ``masks`` is the ascending list
     of mask sizes a best-effort client owns; the last entry is the whole GPU.
-    Kernels go to the smallest mask that holds their profiled CU need; records
-    that are not kernels stay where the client's previous op ran (-1)."""
+    High-priority client idle: the whole GPU.  Request in flight: the smallest
+    mask that holds the kernel's profiled CU need, never the whole GPU when a
+    partial mask exists.  Records that are not kernels stay where the client's
+    previous op ran (-1)."""
     if cls != po.KERNEL:
         return -1
-    if algo != po.ALGO_ORION:
-        return len(masks) - 1
-    for slot, size in enumerate(masks):
-        if sm_used <= size:
+    last = len(masks) - 1
+    if algo != po.ALGO_ORION or not hp_active or last == 0:
+        return last
+    for slot in range(last):
+        if sm_used <= masks[slot]:
             return slot
-    return len(masks) - 1
+    return last - 1
 
 
 class RecordingEnv(po.Env):
     """Wraps another Env; writes both logs while the oracle drives it."""
 
-    def __init__(self, inner, n, masks, ops_of, algo=po.ALGO_ORION):
+    def __init__(self, inner, n, masks, ops_of, algo=po.ALGO_ORION,
+                 hp_active=None):
+        self.hp_active = hp_active    # callable() -> bool: seen[hp] > 0
         self.inner = inner
         self.n = n
         self.masks = list(masks)
@@ -147,7 +152,7 @@ class RecordingEnv(po.Env):
         else:
             cu_slot = place_cu_slot(self.masks, cls,
                                     self.ops_of(client, op_index).sm_used,
-                                    self.algo)
+                                    self.algo, self.hp_active())
         self._dec.append(f"D {client} {owner} {cls} {op_index} {event_slot} "
                          f"{cu_slot}")
         self.inner.dispatch(client, owner, cls, op_index, event_slot)
@@ -264,7 +269,8 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
             env = ReplayEnv(n, polls)
             if rec is None:
                 rec = RecordingEnv(env, n, masks,
-                                   lambda c, k: oracle.ops[c][k])
+                                   lambda c, k: oracle.ops[c][k],
+                                   hp_active=lambda: oracle.seen[n - 1] > 0)
             rec.inner = env
             warmup, witers, algo = bool(int(parts[1])), int(parts[2]), parts[3]
             depth, hp_limit, ustart = int(parts[4]), int(parts[5]), int(parts[6])

@@ -70,7 +70,10 @@ def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
     backend.register_stream(stream)
     with torch.cuda.stream(stream), torch.autograd.set_multithreading_enabled(False):
         with cc.uncaptured(backend):
-            model = BertForQuestionAnswering(bert_config(train)).to(device)
+            with cc.MODEL_INIT_LOCK:
+                cc.seed_everything(seed)
+                model = BertForQuestionAnswering(bert_config(train))
+            model = model.to(device)
             if train:
                 model.train()
                 named = [(n, p) for n, p in model.named_parameters() if "pooler" not in n]
@@ -111,7 +114,7 @@ def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
                 torch.save(state["output"].float().cpu(),
                            os.path.join(save_dir, f"client_{tid}_output.pt"))
             if "loss" in state:
-                res["final_loss"] = float(state["loss"].float().cpu())
+                res["final_loss"] = float(state["loss"].detach().float().cpu())
             return res
 
         with cc.uncaptured(backend):

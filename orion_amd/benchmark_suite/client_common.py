@@ -15,7 +15,15 @@ import torch
 
 from .. import scheduler_frontend as fe
 
+import threading
+
 WARMUP_ITERS = 10     # iterations before the measured run (:188-198, :220)
+
+# Weight initialisation draws from the process-wide generator.  Clients seed it
+# and build their model while holding this lock, so a client's weights do not
+# depend on which other clients share the process (its output can then be
+# compared with its isolated run).
+MODEL_INIT_LOCK = threading.Lock()
 
 
 def seed_everything(seed):

@@ -5,7 +5,7 @@ Counterpart of the reference's ``imagenet_loop``
 (benchmarking/benchmark_suite/train_imagenet.py:71-241): same keyword
 arguments, same loop and barrier protocol, same ``client_{tid}.json``.  Extra,
 optional keys of a job's ``args``: ``dtype`` ("fp32" | "bf16"), ``momentum``,
-``seed``.  Synthetic data follows the job description: images N(0,1), labels
+``seed``, ``deterministic``.  Synthetic data follows the job description: images N(0,1), labels
 uniform over the classes (the reference uses U(0,1) images and all-ones labels,
 :36-37).
 """
@@ -39,8 +39,13 @@ class DummyDataLoader:
 
 def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                   dummy_data, local_rank, barriers, client_barrier, tid,
-                  input_file="", dtype="fp32", momentum=0.9, seed=42):
+                  input_file="", dtype="fp32", momentum=0.9, seed=42,
+                  deterministic=False):
     cc.seed_everything(seed)
+    if deterministic:
+        # keep MIOpen off solvers that accumulate with atomics (split-K), whose
+        # results differ in the last bit from run to run
+        torch.backends.cudnn.deterministic = True
     backend = cc.Backend()
     sleep_times = cc.arrival_gaps(rps, uniform, num_iters, input_file, seed)
     if not dummy_data:
@@ -56,7 +61,10 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
     losses = []
     with torch.cuda.stream(stream), torch.autograd.set_multithreading_enabled(False):
         with cc.uncaptured(backend):
-            model = MODELS[model_name](num_classes=1000).to(device)
+            with cc.MODEL_INIT_LOCK:
+                cc.seed_everything(seed)
+                model = MODELS[model_name](num_classes=1000)
+            model = model.to(device)
             if train:
                 model.train()
                 optimizer = torch.optim.SGD(model.parameters(), lr=0.1, momentum=momentum)
@@ -91,7 +99,7 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                 torch.save(state["output"].float().cpu(),
                            os.path.join(save_dir, f"client_{tid}_output.pt"))
             if "loss" in state:
-                out["final_loss"] = float(state["loss"].float().cpu())
+                out["final_loss"] = float(state["loss"].detach().float().cpu())
             return out
 
         with cc.uncaptured(backend):

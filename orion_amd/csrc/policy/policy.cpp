@@ -115,13 +115,13 @@ bool parse_profile(const std::string& path, std::vector<OpInfo>* ops,
 }
 
 int place_cu_slot(const std::vector<int>& masks, int rec_class, int sm_used,
-                  int algo) {
+                  int algo, bool hp_active) {
   if (rec_class != REC_KERNEL) return -1;
   const int last = (int)masks.size() - 1;
-  if (algo != ALGO_ORION) return last;
-  for (int s = 0; s <= last; ++s)
+  if (algo != ALGO_ORION || !hp_active || last == 0) return last;
+  for (int s = 0; s < last; ++s)
     if (sm_used <= masks[s]) return s;
-  return last;
+  return last - 1;
 }
 
 static int max_sm_used(const std::vector<OpInfo>& ops) {
@@ -171,7 +171,8 @@ void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class) {
     d.cu_slot = 0;  // the high-priority stream spans the whole GPU
   } else {
     d.cu_slot = place_cu_slot(cu_masks_, rec_class,
-                              ops_[client][d.op_index].sm_used, algo_);
+                              ops_[client][d.op_index].sm_used, algo_,
+                              seen_[n_ - 1] > 0);
   }
   host.dispatch(d);
   if (rec_class == REC_KERNEL) {

@@ -54,11 +54,17 @@ struct OpInfo {
 bool parse_profile(const std::string& path, std::vector<OpInfo>* ops,
                    std::string* err);
 
-// CU-mask placement of a best-effort kernel: index of the smallest mask (sizes
-// ascending, last = whole GPU) that holds the op's CU need.  No reference
-// counterpart (the reference owns one stream per client).
+// CU-mask placement of a best-effort kernel (no reference counterpart: the
+// reference owns one stream per client).  `masks` are the sizes, ascending, of
+// the CU-masked streams a best-effort client owns; the last one is the whole
+// GPU.  While the high-priority client is idle a kernel may use the whole GPU.
+// While it has a request in flight the kernel goes to the smallest mask that
+// holds its profiled CU need, and never to the whole-GPU stream when a partial
+// mask exists: the compute units outside the widest partial mask stay free for
+// the high-priority client.  Records that are not kernels stay where the
+// client's work is (-1).
 int place_cu_slot(const std::vector<int>& masks, int rec_class, int sm_used,
-                  int algo);
+                  int algo, bool hp_active);
 
 struct Dispatch {
   int client;      // whose record

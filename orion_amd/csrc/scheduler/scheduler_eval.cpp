@@ -122,6 +122,7 @@ class LiveHost : public PolicyHost {
     update_valid_ = false;
   }
   void begin_phase() {
+    last_progress_ = Clock::now();
     for (int i = 0; i < n_; ++i) first_start_[(size_t)i] = Clock::time_point();
     phase_start_ = Clock::now();
   }
@@ -224,6 +225,7 @@ class LiveHost : public PolicyHost {
       }
     }
     ++dispatched_[(size_t)d.client];
+    last_progress_ = Clock::now();
     // pop_from_queue: retiring the record releases the caller
     ch.head.store(head + 1, std::memory_order_release);
   }
@@ -234,6 +236,7 @@ class LiveHost : public PolicyHost {
     const float ms = (float)iteration_us(client) / 1000.0f;
     durations_ms_[(size_t)client].push_back(ms);
     start_pending_[(size_t)client] = true;
+    last_progress_ = Clock::now();
     if (client == update_owner_) update_valid_ = false;
   }
 
@@ -243,36 +246,38 @@ class LiveHost : public PolicyHost {
 
  private:
   // The reference spins forever when a client's kernel count disagrees with its
-  // profile (scheduler_eval.cpp:282, :389).  Here that state -- the client
-  // waits in block() with an empty queue while the policy still expects more
-  // kernels -- is reported and ends the process once it has lasted a while.
+  // profile, or when a client dies mid-iteration (scheduler_eval.cpp:282, :389).
+  // Here a scheduler that has neither dispatched nor completed anything for a
+  // while, although a client waits in block() or holds a queued record, reports
+  // what it sees and ends the process.
   void watchdog() {
     if (!policy_) return;
     const auto now = Clock::now();
+    if (std::chrono::duration<double>(now - last_progress_).count() < stuck_limit_s_) return;
+    bool someone_waits = false;
+    std::string dump;
     for (int i = 0; i < n_; ++i) {
       ClientChannel& ch = cap_->channels[i];
-      const bool waiting = ch.block_calls.load(std::memory_order_acquire) >
-                           ch.released_iters.load(std::memory_order_acquire);
-      const bool empty = ch.tail.load(std::memory_order_acquire) ==
-                         ch.head.load(std::memory_order_acquire);
-      const int seen = policy_->seen()[(size_t)i];
-      const int want = policy_->num_kernels()[(size_t)i];
-      if (waiting && empty && seen != want && seen != 0) {
-        if (stuck_since_.size() != (size_t)n_) stuck_since_.assign((size_t)n_, Clock::time_point());
-        if (stuck_since_[(size_t)i] == Clock::time_point()) {
-          stuck_since_[(size_t)i] = now;
-        } else if (std::chrono::duration<double>(now - stuck_since_[(size_t)i]).count() > stuck_limit_s_) {
-          char msg[256];
-          snprintf(msg, sizeof msg,
-                   "client %d submitted %d kernel records in this iteration and waits in "
-                   "block(), but its profile names %d (num_kernels): the job file and the "
-                   "profile do not match this client", i, seen, want);
-          die(msg);
-        }
-      } else if (stuck_since_.size() == (size_t)n_) {
-        stuck_since_[(size_t)i] = Clock::time_point();
-      }
+      const long long blocked = ch.block_calls.load(std::memory_order_acquire);
+      const long long released = ch.released_iters.load(std::memory_order_acquire);
+      const unsigned long long queued = ch.tail.load(std::memory_order_acquire) -
+                                        ch.head.load(std::memory_order_acquire);
+      if (blocked > released || queued > 0) someone_waits = true;
+      char line[256];
+      snprintf(line, sizeof line,
+               "\n  client %d: %d of %d kernel records seen this iteration, %llu queued, "
+               "block() calls %lld, iterations released %lld, iterations done %d", i,
+               policy_->seen()[(size_t)i], policy_->num_kernels()[(size_t)i], queued, blocked,
+               released, policy_->cur_iters()[(size_t)i]);
+      dump += line;
     }
+    if (!someone_waits) {
+      last_progress_ = now;
+      return;
+    }
+    die("no dispatch and no completed iteration for " + std::to_string((int)stuck_limit_s_) +
+        " s while clients wait; a client's kernel count probably differs from its profile's "
+        "num_kernels, or a client died:" + dump);
   }
 
   void create_streams() {
@@ -312,7 +317,7 @@ class LiveHost : public PolicyHost {
   std::vector<int> masks_;
   const Policy* policy_ = nullptr;
   uint64_t polls_ = 0;
-  std::vector<Clock::time_point> stuck_since_;
+  Clock::time_point last_progress_ = Clock::now();
   double stuck_limit_s_ = getenv("ORION_STUCK_LIMIT_S") ? atof(getenv("ORION_STUCK_LIMIT_S")) : 20.0;
   const HipApi* hip_;
   CaptureState* cap_;

@@ -78,7 +78,15 @@ def launch_jobs(config_dict_list, input_args, run_eval=True, function_dict=None,
                            "tid": i})
 
         def target(func=func, kwargs=model_args, i=i):
-            results[i] = func(**kwargs)
+            try:
+                results[i] = func(**kwargs)
+            except BaseException:
+                # A dead client would leave the scheduler polling for records
+                # that never come (the reference hangs): end the job loudly.
+                import traceback
+                traceback.print_exc()
+                print(f"orion: client {i} failed; aborting the job", flush=True)
+                os._exit(1)
 
         thread = threading.Thread(target=target, name=f"orion-client-{i}")
         thread.start()

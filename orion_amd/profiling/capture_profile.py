@@ -76,7 +76,16 @@ def capture(entry, out_prefix, iters=14, function_dict=None):
     # a profile run must not pace itself: closed loop
     kwargs["rps"] = 0
     os.environ.setdefault("ORION_RESULT_DIR", os.path.dirname(out_prefix) or ".")
-    thread = threading.Thread(target=function_dict[entry["arch"]], kwargs=kwargs)
+    def target():
+        try:
+            function_dict[entry["arch"]](**kwargs)
+        except BaseException:
+            import traceback
+            traceback.print_exc()
+            print("orion: the profiled client failed; aborting", flush=True)
+            os._exit(1)
+
+    thread = threading.Thread(target=target)
     thread.start()
     trace_path = out_prefix + ".trace.csv"
     rc = sched.orion_profile_begin(thread.native_id, trace_path.encode())

@@ -1,0 +1,109 @@
+"""The whole hot path on a real MI355X: interception (LD_PRELOAD) -> queues ->
+policy -> CU-masked dispatch, in child processes started the way a user starts
+the launcher.
+
+* every client's output equals its isolated run, bit for bit (same kernels);
+* the model client's output is within 1e-3 (relative to the largest reference
+  magnitude) of the PyTorch CPU fp32 reference -- the tolerance the job
+  description names for floating point;
+* the dispatch-decision sequence the live scheduler recorded is reproduced
+  byte for byte by the CPU oracle and by the native core replaying the recorded
+  observations over the same profile files.
+"""
+
+import copy
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import obslog
+from tests import jobs
+
+pytestmark = pytest.mark.gpu
+CPU_RTOL = 1e-3
+
+
+def _check_replay(record_dir):
+    obs = open(os.path.join(record_dir, "observations.log")).read()
+    dec = open(os.path.join(record_dir, "decisions.log")).read()
+    assert dec.count("\nD ") > 50
+    assert jobs.native_replay(obs) == dec
+    assert obslog.replay(obs) == dec
+    return dec
+
+
+def test_kernel_pair_through_the_scheduler(tmp_path):
+    from orion_amd import kernel_pair
+    res = kernel_pair.run_child(small=True, check=True, workdir=str(tmp_path), hp_iters=80)
+    assert res["outputs_match"]
+    assert res["hp_colocated"]["iterations"] == 80
+    assert res["be_colocated"]["iterations"] > 10
+    dec = _check_replay(os.path.join(str(tmp_path), "out_co"))
+    # best-effort kernels were dispatched on masked slots while HP was active
+    be_slots = {l.split()[6] for l in dec.splitlines() if l.startswith("D 0 0 k")}
+    assert be_slots & {"0", "1", "2"} and "3" in be_slots
+    # the triad's output is b + s*c for the inputs the client seeds
+    out = torch.load(os.path.join(str(tmp_path), "out_co", "client_0_output.pt"),
+                     weights_only=True)
+    b, c = kernel_pair._inputs_triad(1 << 22, "cuda:0")
+    want = torch.addcmul(b[:4096].double(), c[:4096].double(),
+                         torch.tensor(float(torch.tensor(1.7, dtype=torch.float32)),
+                                      dtype=torch.float64, device="cuda:0")).float().cpu()
+    assert torch.equal(out, want)
+
+
+def test_resnet50_colocation_outputs_and_replay(tmp_path):
+    from orion_amd import colocate
+    from orion_amd.benchmark_suite.vision_models import resnet50
+    from orion_amd.profiling import capture_profile
+    work = str(tmp_path)
+    job = [
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": True, "deterministic": True}},
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 40,
+         "args": {"model_name": "resnet50", "batchsize": 4, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": False, "dtype": "fp32",
+                  "deterministic": True}},
+    ]
+    cfg = os.path.join(work, "job.json")
+    with open(cfg, "w") as f:
+        json.dump(job, f)
+    env = colocate.preload_env()
+    os.environ["LD_PRELOAD"] = env["LD_PRELOAD"]
+    try:
+        filled = capture_profile.fill_job(cfg, os.path.join(work, "profiles"),
+                                          os.path.join(work, "filled.json"))
+    finally:
+        os.environ["LD_PRELOAD"] = ":".join(
+            p for p in env["LD_PRELOAD"].split(":") if "libinttemp.so" not in p)
+    iso_dir, co_dir = os.path.join(work, "iso_out"), os.path.join(work, "co_out")
+    os.makedirs(iso_dir)
+    os.makedirs(co_dir)
+    colocate.run_job([copy.deepcopy(filled[-1])], "orion", os.path.join(work, "iso"),
+                     160000, env={"ORION_SAVE_OUTPUT_DIR": iso_dir})
+    co = colocate.run_job(copy.deepcopy(filled), "orion", os.path.join(work, "co"),
+                          160000, env={"ORION_SAVE_OUTPUT_DIR": co_dir,
+                                       "ORION_RECORD_DIR": co_dir})
+    assert co[-1]["iterations"] == 40 and co[0]["iterations"] >= 10
+    iso_out = torch.load(os.path.join(iso_dir, "client_0_output.pt"), weights_only=True)
+    co_out = torch.load(os.path.join(co_dir, "client_1_output.pt"), weights_only=True)
+    # Same kernels, deterministic solvers: bit-exact.  (Without the
+    # deterministic flag MIOpen may pick split-K kernels that accumulate with
+    # atomics and differ in the last bit between any two runs.)
+    assert torch.equal(iso_out, co_out), float((iso_out - co_out).abs().max())
+
+    # PyTorch CPU fp32 reference of the same model and input
+    from orion_amd.benchmark_suite import client_common as cc
+    from orion_amd.benchmark_suite.train_imagenet import DummyDataLoader
+    with cc.MODEL_INIT_LOCK:
+        cc.seed_everything(42)
+        model = resnet50().eval()
+    data, _ = next(DummyDataLoader(4, 42))
+    with torch.no_grad():
+        ref = model(data.float())
+    err = (co_out - ref).abs().max() / ref.abs().max()
+    assert err <= CPU_RTOL, float(err)
+    _check_replay(co_dir)

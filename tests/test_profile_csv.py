@@ -150,10 +150,18 @@ def test_cu_slot_placement_matches_oracle():
                                     po.ALGO_SEQUENTIAL]):
         for cls in po.ALL_CLASSES:
             for sm in [0, 1, 32, 33, 64, 65, 128, 129, 256, 257, 12544]:
-                want = obslog.place_cu_slot(masks, cls, sm, algo)
-                got = lib.orion_place_cu_slot(arr, 4, cls_id[cls], sm, algo_id)
-                assert got == want
-    # hand-worked: smallest mask that holds the need, whole GPU beyond
-    assert obslog.place_cu_slot(masks, po.KERNEL, 33, po.ALGO_ORION) == 1
-    assert obslog.place_cu_slot(masks, po.KERNEL, 4000, po.ALGO_ORION) == 3
-    assert obslog.place_cu_slot(masks, po.MEMCPY, 1, po.ALGO_ORION) == -1
+                for active in (False, True):
+                    want = obslog.place_cu_slot(masks, cls, sm, algo, active)
+                    got = lib.orion_place_cu_slot(arr, 4, cls_id[cls], sm, algo_id,
+                                                  int(active))
+                    assert got == want
+    # hand-worked: idle -> whole GPU; active -> smallest mask that holds the
+    # need, capped below the whole GPU; a single mask leaves no choice
+    place = obslog.place_cu_slot
+    assert place(masks, po.KERNEL, 33, po.ALGO_ORION, False) == 3
+    assert place(masks, po.KERNEL, 33, po.ALGO_ORION, True) == 1
+    assert place(masks, po.KERNEL, 4000, po.ALGO_ORION, True) == 2
+    assert place(masks, po.KERNEL, 1, po.ALGO_ORION, True) == 0
+    assert place(masks, po.MEMCPY, 1, po.ALGO_ORION, True) == -1
+    assert place([256], po.KERNEL, 4000, po.ALGO_ORION, True) == 0
+    assert place(masks, po.KERNEL, 1, po.ALGO_REEF, True) == 3
