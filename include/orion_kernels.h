@@ -27,8 +27,10 @@ enum orion_status {
 
 /* a[i] = fmaf(s, c[i], b[i]) for i in [0, n): one fused multiply-add per
  * element, so results are bit-identical to C's fmaf on the host.
- * grid_blocks <= 0 selects the default grid (2048 workgroups of 256 lanes,
- * fewer for small n); any positive value is honoured (grid-stride loop).
+ * grid_blocks <= 0 selects the default launch (one 16-byte access per lane,
+ * n / 1024 workgroups of 256 lanes); a smaller positive value is honoured with
+ * block-contiguous chunks.  ORION_ERR_SHAPE if n needs more than 2^31 - 1
+ * workgroups.
  * Memory-bound stand-in for bnorm_trainer.py:20-27 of the reference. */
 int orion_triad_f32(float* a, const float* b, const float* c, float s,
                     size_t n, int grid_blocks, void* stream);
@@ -37,7 +39,7 @@ int orion_triad_f32(float* a, const float* b, const float* c, float s,
  * both K-contiguous (row-major A, row-major B = the weight layout of a linear
  * layer).  Accumulation is fp32 on the matrix cores; C is fp32 when
  * out_is_f32 != 0, else bf16 rounded to nearest even.  Requires M % 256 == 0,
- * N % 256 == 0, K % 64 == 0 (ORION_ERR_SHAPE otherwise).
+ * N % 256 == 0, K % 32 == 0 (ORION_ERR_SHAPE otherwise).
  * Compute-bound stand-in for conv_trainer.py:20-27 of the reference. */
 int orion_gemm_bf16_nt(const void* A, const void* B, void* C, int M, int N,
                        int K, int out_is_f32, void* stream);

@@ -1,0 +1,132 @@
+// Native driver for the two co-location kernels, for profiler runs
+// (rocprofv3 --kernel-trace / --pmc -- orion_amd/bench_kernels): it uses the
+// system HIP runtime only, so a profiler sees exactly these kernels.
+//
+//   bench_kernels [--reps N] [--gemm-n N] [--triad-elems N] [--mask CUS]
+//
+// Per kernel it prints the average launch duration measured with HIP events on
+// the stream the kernel runs on, and the achieved rate against its roofline.
+// A plain 16-byte-per-lane copy kernel of known size runs as well: its
+// FETCH_SIZE / WRITE_SIZE readings give the factor that scales the counters of
+// the other kernels to bytes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "orion_kernels.h"
+
+#define CHECK(x)                                                              \
+  do {                                                                        \
+    hipError_t e_ = (x);                                                      \
+    if (e_ != hipSuccess) {                                                   \
+      fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #x, hipGetErrorString(e_)); \
+      exit(1);                                                                \
+    }                                                                         \
+  } while (0)
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// uniform(-1, 1) from a counter hash; fp32 or bf16 (upper half) output
+__global__ void init_uniform(uint32_t* out, size_t n, uint32_t seed, int as_bf16_pairs) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    uint32_t x = (uint32_t)i * 2654435761u + seed;
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    float f = (float)(x >> 8) * (2.0f / 16777216.0f) - 1.0f;
+    uint32_t bits = __builtin_bit_cast(uint32_t, f);
+    if (as_bf16_pairs) {
+      uint32_t y = x * 747796405u + 2891336453u;
+      float g = (float)(y >> 8) * (2.0f / 16777216.0f) - 1.0f;
+      out[i] = (bits >> 16) | (__builtin_bit_cast(uint32_t, g) & 0xffff0000u);
+    } else {
+      out[i] = bits;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_f32x4_kernel(f32x4* __restrict__ dst,
+                                                         const f32x4* __restrict__ src,
+                                                         size_t n_vec4) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * 256;
+  for (; i < n_vec4; i += stride) dst[i] = src[i];
+}
+
+static float time_ms(hipStream_t s, int reps, int warmup, void (*launch)(hipStream_t, void*), void* ctx) {
+  hipEvent_t a, b;
+  CHECK(hipEventCreate(&a));
+  CHECK(hipEventCreate(&b));
+  for (int i = 0; i < warmup; ++i) launch(s, ctx);
+  CHECK(hipEventRecord(a, s));
+  for (int i = 0; i < reps; ++i) launch(s, ctx);
+  CHECK(hipEventRecord(b, s));
+  CHECK(hipEventSynchronize(b));
+  float ms = 0;
+  CHECK(hipEventElapsedTime(&ms, a, b));
+  CHECK(hipEventDestroy(a));
+  CHECK(hipEventDestroy(b));
+  return ms / reps;
+}
+
+struct GemmCtx { void *A, *B, *C; int n; };
+struct TriadCtx { float *a, *b, *c; size_t n; };
+
+static void launch_gemm(hipStream_t s, void* p) {
+  GemmCtx* g = (GemmCtx*)p;
+  if (orion_gemm_bf16_nt(g->A, g->B, g->C, g->n, g->n, g->n, 0, s) != ORION_OK) exit(2);
+}
+static void launch_triad(hipStream_t s, void* p) {
+  TriadCtx* t = (TriadCtx*)p;
+  if (orion_triad_f32(t->a, t->b, t->c, 1.7f, t->n, 0, s) != ORION_OK) exit(2);
+}
+static void launch_copy(hipStream_t s, void* p) {
+  TriadCtx* t = (TriadCtx*)p;
+  hipLaunchKernelGGL(copy_f32x4_kernel, dim3(2048), dim3(256), 0, s, (f32x4*)t->a,
+                     (const f32x4*)t->b, t->n / 4);
+}
+
+int main(int argc, char** argv) {
+  int reps = 20, gemm_n = 8192, mask = 0;
+  size_t elems = (size_t)1 << 28;
+  for (int i = 1; i + 1 < argc; i += 2) {
+    if (!strcmp(argv[i], "--reps")) reps = atoi(argv[i + 1]);
+    else if (!strcmp(argv[i], "--gemm-n")) gemm_n = atoi(argv[i + 1]);
+    else if (!strcmp(argv[i], "--triad-elems")) elems = strtoull(argv[i + 1], nullptr, 10);
+    else if (!strcmp(argv[i], "--mask")) mask = atoi(argv[i + 1]);
+  }
+  hipStream_t full = nullptr, masked = nullptr;
+  if (orion_stream_create(0, (void**)&full) != ORION_OK) return 3;
+  if (orion_stream_create(mask, (void**)&masked) != ORION_OK) return 3;
+
+  GemmCtx g;
+  g.n = gemm_n;
+  const size_t mat = (size_t)gemm_n * gemm_n;
+  CHECK(hipMalloc(&g.A, mat * 2));
+  CHECK(hipMalloc(&g.B, mat * 2));
+  CHECK(hipMalloc(&g.C, mat * 2));
+  hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)g.A, mat / 2, 1u, 1);
+  hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)g.B, mat / 2, 2u, 1);
+  TriadCtx t;
+  t.n = elems;
+  CHECK(hipMalloc((void**)&t.a, elems * 4));
+  CHECK(hipMalloc((void**)&t.b, elems * 4));
+  CHECK(hipMalloc((void**)&t.c, elems * 4));
+  hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)t.b, elems, 3u, 0);
+  hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)t.c, elems, 4u, 0);
+  CHECK(hipStreamSynchronize(full));
+
+  const float gemm_ms = time_ms(full, reps, 3, launch_gemm, &g);
+  const float triad_ms = time_ms(masked, reps, 3, launch_triad, &t);
+  const float copy_ms = time_ms(full, reps, 3, launch_copy, &t);
+  const double flops = 2.0 * gemm_n * (double)gemm_n * gemm_n;
+  printf("{\"reps\": %d, \"gemm\": {\"n\": %d, \"ms\": %.5f, \"tflops\": %.2f, \"frac_of_2500\": %.4f}, "
+         "\"triad\": {\"elems\": %zu, \"cu_mask\": %d, \"ms\": %.5f, \"gbs\": %.1f, \"frac_of_8000\": %.4f}, "
+         "\"copy\": {\"bytes\": %zu, \"ms\": %.5f, \"gbs\": %.1f}}\n",
+         reps, gemm_n, gemm_ms, flops / gemm_ms / 1e9, flops / gemm_ms / 1e9 / 2500.0, elems,
+         mask, triad_ms, 12.0 * elems / triad_ms / 1e6, 12.0 * elems / triad_ms / 1e6 / 8000.0,
+         elems * 8, copy_ms, 8.0 * elems / copy_ms / 1e6);
+  return 0;
+}
