@@ -31,6 +31,10 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# profiles/bench_kernels_gemm8192_triad1GiB_counters.txt
+GEMM_TRAFFIC_BYTES = int((791052.6 * 2.0 + 134048.9 * 1.0) * 1024)
+TRIAD_TRAFFIC_BYTES = int((1048588.2 * 2.0 + 1048576.0 * 1.0) * 1024)
+
 METRIC = "HP p99 latency vs isolated + BE iters/sec retained, co-located on 1 MI355X"
 WORKLOAD = ("HP: ResNet-50 inference, batch 4, bf16, Poisson arrivals at 80 req/s, inputs "
             "4x3x224x224 N(0,1); BE: ResNet-50 training, batch 32, SGD momentum 0.9, "
@@ -182,13 +186,16 @@ def main():
     out["roofline"] = {"kernel": "gemm_bf16_nt_kernel<bf16 out> 8192x8192x8192", "bound": "mfma",
                        "achieved": gemm["tflops"], "peak": kp.MFMA_BF16_PEAK_TFLOPS,
                        "unit": "TFLOP/s", "frac": gemm["tflops"] / kp.MFMA_BF16_PEAK_TFLOPS,
-                       "flops_per_launch": flops, "ms_per_launch": gemm["ms"], "traffic": None}
+                       "flops_per_launch": flops, "ms_per_launch": gemm["ms"],
+                       # bytes past the L2s per launch, from the committed rocprofv3
+                       # FETCH_SIZE / WRITE_SIZE runs (scaled by a copy kernel)
+                       "traffic": GEMM_TRAFFIC_BYTES}
     tri = alone["triad"]["256"]
     out["roofline_triad"] = {"kernel": "triad_f32_kernel 3 x 1 GiB", "bound": "hbm",
                              "achieved": tri["gbs"], "peak": kp.HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": tri["gbs"] / kp.HBM_PEAK_GBS,
                              "bytes_per_launch": 12 * kp.TRIAD_ELEMS,
-                             "ms_per_launch": tri["ms"], "traffic": None}
+                             "ms_per_launch": tri["ms"], "traffic": TRIAD_TRAFFIC_BYTES}
     out["kernel_pair"] = {
         "workload": "configs[1]: HP bf16 GEMM 8192^3 beside BE fp32 triad over 1 GiB arrays",
         "triad_alone_gbs_by_cu_mask": {k: v["gbs"] for k, v in alone["triad"].items()},
