@@ -62,7 +62,7 @@ def colocation(steps, workdir, max_be_duration, masks):
     os.environ.update({k: v for k, v in colocate.preload_env().items()
                        if k == "LD_PRELOAD"})
     job = capture_profile.fill_job(cfg, os.path.join(workdir, "profiles"),
-                                   os.path.join(workdir, "job_filled.json"))
+                                   os.path.join(workdir, "job_filled.json"), quiet=True)
     env = {"ORION_RECORD_DIR": os.path.join(workdir, "colocated")}
     if masks:
         env["ORION_BE_CU_MASKS"] = masks

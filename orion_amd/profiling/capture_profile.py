@@ -131,7 +131,7 @@ def profile_name(entry):
     return f"{a.get('model_name', entry['arch'])}_{a['batchsize']}_{a.get('dtype', 'fp32')}_{phase}"
 
 
-def fill_job(config_path, out_dir, filled_path, iters=14):
+def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False):
     """Profile every client of a job file, each alone in a process of its own,
     and write a copy of the job file with kernel_file / num_kernels (and the
     additional_* pair) filled in."""
@@ -144,9 +144,14 @@ def fill_job(config_path, out_dir, filled_path, iters=14):
     for idx, entry in enumerate(job):
         prefix = os.path.abspath(os.path.join(out_dir, profile_name(entry)))
         if prefix not in done:
-            subprocess.run([sys.executable, "-m", "orion_amd.profiling.capture_profile",
-                            "--config", config_path, "--client", str(idx), "--out",
-                            prefix, "--iters", str(iters)], check=True)
+            cmd = [sys.executable, "-m", "orion_amd.profiling.capture_profile",
+                   "--config", config_path, "--client", str(idx), "--out", prefix,
+                   "--iters", str(iters)]
+            if quiet:     # keep the caller's stdout clean; the log stays beside the profile
+                with open(prefix + ".log", "w") as log:
+                    subprocess.run(cmd, check=True, stdout=log, stderr=subprocess.STDOUT)
+            else:
+                subprocess.run(cmd, check=True)
             with open(prefix + ".json") as f:
                 done[prefix] = json.load(f)
         summary = done[prefix]
