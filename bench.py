@@ -52,7 +52,7 @@ def c3_job(hp_iters):
     ]
 
 
-def colocation(steps, workdir, max_be_duration, masks):
+def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False):
     from orion_amd import colocate
     from orion_amd.profiling import capture_profile
     cfg = os.path.join(workdir, "job.json")
@@ -62,7 +62,8 @@ def colocation(steps, workdir, max_be_duration, masks):
     os.environ.update({k: v for k, v in colocate.preload_env().items()
                        if k == "LD_PRELOAD"})
     job = capture_profile.fill_job(cfg, os.path.join(workdir, "profiles"),
-                                   os.path.join(workdir, "job_filled.json"), quiet=True)
+                                   os.path.join(workdir, "job_filled.json"), quiet=True,
+                                   use_rocprof=use_rocprof)
     env = {"ORION_RECORD_DIR": os.path.join(workdir, "colocated")}
     if masks:
         env["ORION_BE_CU_MASKS"] = masks
@@ -142,6 +143,9 @@ def main():
                          "(artifact_evaluation/fig7/run_orion.py:6-15)")
     ap.add_argument("--be-cu-masks", default="",
                     help="override ORION_BE_CU_MASKS for the co-located run")
+    ap.add_argument("--rocprof-profiles", action="store_true",
+                    help="take the profiles' class, duration and register columns from "
+                         "rocprofv3 runs (adds about two minutes)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="only the in-process kernel measurements (for profiler runs: "
                          "starts no child process)")
@@ -162,7 +166,8 @@ def main():
                       "algo": "orion", "max_be_duration_ns": args.max_be_duration}}
     if not args.kernels_only:
         t0 = time.time()
-        co = colocation(args.steps, workdir, args.max_be_duration, args.be_cu_masks)
+        co = colocation(args.steps, workdir, args.max_be_duration, args.be_cu_masks,
+                        args.rocprof_profiles)
         out["value"] = co["hp_p99_ratio"]
         out["ms_per_step"] = 1000.0 / co["hp_colocated"]["throughput"]
         out["hp"] = {"isolated_ms": {k: co["hp_isolated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},

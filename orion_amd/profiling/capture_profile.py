@@ -131,7 +131,7 @@ def profile_name(entry):
     return f"{a.get('model_name', entry['arch'])}_{a['batchsize']}_{a.get('dtype', 'fp32')}_{phase}"
 
 
-def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False):
+def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False, use_rocprof=False):
     """Profile every client of a job file, each alone in a process of its own,
     and write a copy of the job file with kernel_file / num_kernels (and the
     additional_* pair) filled in."""
@@ -154,6 +154,20 @@ def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False):
                 subprocess.run(cmd, check=True)
             with open(prefix + ".json") as f:
                 done[prefix] = json.load(f)
+            if use_rocprof:
+                # bound class, durations and register counts from rocprofv3
+                from . import rocprof
+                summary = done[prefix]
+                steady = summary.get("additional_kernel_file", summary["kernel_file"])
+                rdir = prefix + ".rocprof"
+                rocprof.collect(config_path, idx, rdir)
+                stats = rocprof.merge(steady, rdir, steady)
+                if "additional_kernel_file" in summary:
+                    import shutil
+                    shutil.copyfile(steady, summary["kernel_file"])
+                summary["rocprof"] = stats
+                with open(prefix + ".json", "w") as f:
+                    json.dump(summary, f, indent=1)
         summary = done[prefix]
         for key in ("kernel_file", "num_kernels", "additional_kernel_file",
                     "additional_num_kernels"):
@@ -174,9 +188,12 @@ def main(argv=None):
     p.add_argument("--fill", help="profile every client and write the completed "
                                   "job file here (profiles go to --out-dir)")
     p.add_argument("--out-dir", default="profiles_gfx950")
+    p.add_argument("--rocprof", action="store_true",
+                   help="with --fill: also run rocprofv3 and take class, duration and "
+                        "register counts from it")
     a = p.parse_args(argv)
     if a.fill:
-        fill_job(a.config, a.out_dir, a.fill, a.iters)
+        fill_job(a.config, a.out_dir, a.fill, a.iters, use_rocprof=a.rocprof)
         return
     import torch
     torch.cuda.set_device(0)

@@ -74,3 +74,38 @@ def classify(name, hbm_fraction=None, mfma_fraction=None, threshold=0.6):
     if any(h in low for h in MEMORY_HINTS):
         return 0
     return -1
+
+
+# MI355X peaks used to place a kernel on the roofline
+PEAK_HBM_BYTES_PER_S = 8.0e12
+PEAK_VECTOR_FP32_FLOPS = 157.3e12
+PEAK_VECTOR_FP16_FLOPS = 314.6e12       # packed half rate
+PEAK_MFMA_FP32_FLOPS = 157.3e12
+PEAK_MFMA_BF16_FLOPS = 2.5e15
+
+
+def classify_roofline(bytes_moved, vector_fp32_flops=0.0, vector_fp16_flops=0.0,
+                      mfma_fp32_flops=0.0, mfma_bf16_flops=0.0, hbm_fraction=None,
+                      mfma_fraction=None, threshold=0.6):
+    """The reference's rule (profiling/postprocessing/roofline_analysis.py:37-71)
+    on MI355X terms.  A kernel that executes floating-point instructions is
+    compute-bound (1) when its arithmetic intensity lies right of the roofline's
+    knee, else memory-bound (0); because the knee differs per instruction type
+    here (matrix cores vs vector ALU), the comparison is done in time: the
+    shortest time the flops could take at peak against the shortest time the
+    bytes could take at peak.  A kernel without floating-point instructions falls
+    back to utilisation (>= 60 % of the matrix cores -> 1, >= 60 % of HBM
+    bandwidth -> 0), else unknown (-1)."""
+    flops = vector_fp32_flops + vector_fp16_flops + mfma_fp32_flops + mfma_bf16_flops
+    if flops > 0:
+        t_compute = (vector_fp32_flops / PEAK_VECTOR_FP32_FLOPS
+                     + vector_fp16_flops / PEAK_VECTOR_FP16_FLOPS
+                     + mfma_fp32_flops / PEAK_MFMA_FP32_FLOPS
+                     + mfma_bf16_flops / PEAK_MFMA_BF16_FLOPS)
+        t_memory = bytes_moved / PEAK_HBM_BYTES_PER_S
+        return 1 if t_compute > t_memory else 0
+    if mfma_fraction is not None and mfma_fraction >= threshold:
+        return 1
+    if hbm_fraction is not None and hbm_fraction >= threshold:
+        return 0
+    return -1
