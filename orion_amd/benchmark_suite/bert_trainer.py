@@ -25,7 +25,8 @@ VOCAB = 30522
 
 
 def bert_config(train):
-    from transformers import BertConfig
+    with cc.MODEL_INIT_LOCK:   # re-entrant; transformers' lazy imports are not thread-safe
+        from transformers import BertConfig
     vocab = VOCAB + (8 - VOCAB % 8) % 8
     if train:
         return BertConfig(vocab_size=vocab, hidden_size=768, num_hidden_layers=12,
@@ -56,7 +57,8 @@ class DummyDataLoader:
 
 def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
               barriers, client_barrier, tid, dtype="fp32", seed=42):
-    from transformers import BertForQuestionAnswering
+    with cc.MODEL_INIT_LOCK:   # transformers' lazy imports are not thread-safe
+        from transformers import BertForQuestionAnswering
     cc.seed_everything(seed)
     backend = cc.Backend()
     sleep_times = cc.arrival_gaps(rps, uniform, num_iters, "", seed)

@@ -23,7 +23,7 @@ WARMUP_ITERS = 10     # iterations before the measured run (:188-198, :220)
 # and build their model while holding this lock, so a client's weights do not
 # depend on which other clients share the process (its output can then be
 # compared with its isolated run).
-MODEL_INIT_LOCK = threading.Lock()
+MODEL_INIT_LOCK = threading.RLock()
 
 
 def seed_everything(seed):

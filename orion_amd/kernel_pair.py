@@ -186,7 +186,7 @@ def pair_job(small=False, hp_iters=60, rps=0):
 
 
 def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
-              max_be_duration=1_000_000):
+              max_be_duration=1_000_000, algo="orion", reef_depth=12):
     """Profile both clients and run the pair isolated and co-located, in child
     processes with the interception library preloaded.  Returns the experiment
     summary (see ``colocate.experiment``) plus ``outputs_match`` when ``check``."""
@@ -226,7 +226,8 @@ def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
     if check:
         e["ORION_SAVE_OUTPUT_DIR"] = os.path.join(workdir, "out_co")
         e["ORION_RECORD_DIR"] = os.path.join(workdir, "out_co")
-    co = colocate.run_job(job, "orion", os.path.join(workdir, "co"), max_be_duration, env=e)
+    co = colocate.run_job(job, algo, os.path.join(workdir, "co"), max_be_duration,
+                          reef_depth=reef_depth, env=e)
     res["hp_colocated"], res["be_colocated"] = co[-1], co[0]
     res["be_retained"] = co[0]["throughput"] / res["be_isolated"]["throughput"]
     if check:

@@ -54,6 +54,20 @@ def test_kernel_pair_through_the_scheduler(tmp_path):
     assert torch.equal(out, want)
 
 
+@pytest.mark.parametrize("algo", ["reef", "sequential"])
+def test_other_policies_on_the_gpu(tmp_path, algo):
+    """--algo reef / sequential (reference: scheduler_eval.cpp:93-236) through
+    the same path: outputs unchanged, recorded decisions replayed bit-exactly."""
+    from orion_amd import kernel_pair
+    res = kernel_pair.run_child(small=True, check=True, workdir=str(tmp_path), hp_iters=60,
+                                algo=algo, reef_depth=4)
+    assert res["outputs_match"]
+    assert res["hp_colocated"]["iterations"] == 60
+    dec = _check_replay(os.path.join(str(tmp_path), "out_co"))
+    if algo == "sequential":      # everything runs on the first client's stream set
+        assert all(l.split()[2] == "0" for l in dec.splitlines() if l.startswith("D "))
+
+
 def test_resnet50_colocation_outputs_and_replay(tmp_path):
     from orion_amd import colocate
     from orion_amd.benchmark_suite.vision_models import resnet50
