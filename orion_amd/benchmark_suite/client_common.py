@@ -79,7 +79,14 @@ class Backend:
         self.lib = fe.load_capture_library()
 
     def block(self, it):
-        self.lib.block(it)
+        """Wait until iteration ``it`` has completed on the GPU.  Under the
+        scheduler that is libinttemp's block(); when the calling thread is not a
+        scheduled client (stand-alone runs) the current stream is synchronised
+        instead, so the loop measures the same thing either way."""
+        if self.lib.orion_client_index() >= 0:
+            self.lib.block(it)
+        elif torch.cuda.is_available():
+            torch.cuda.current_stream().synchronize()
 
     def stop(self):
         return bool(self.lib.stop())
