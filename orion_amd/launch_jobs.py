@@ -47,6 +47,27 @@ def check_preloaded():
             f"LD_PRELOAD={_lib.CAPTURE_LIB} (append to any value already set)")
 
 
+def job_lists(config_dict_list):
+    """The per-client lists the scheduler front end takes, from a job file
+    (reference: launch_jobs.py:68-75).  The LAST entry is the high-priority
+    client (scheduler_eval.cpp:256)."""
+    for c in config_dict_list:
+        for key in ("arch", "kernel_file", "num_kernels", "num_iters", "args"):
+            if key not in c:
+                raise KeyError(f"job entry lacks {key!r}: {c}")
+        if "train" not in c["args"]:
+            raise KeyError("job entry args lack 'train'")
+    return {
+        "model_names": [c["arch"] for c in config_dict_list],
+        "model_files": [c["kernel_file"] for c in config_dict_list],
+        "additional_model_files": [c.get("additional_kernel_file") for c in config_dict_list],
+        "num_kernels": [c["num_kernels"] for c in config_dict_list],
+        "num_iters": [c["num_iters"] for c in config_dict_list],
+        "train_list": [c["args"]["train"] for c in config_dict_list],
+        "additional_num_kernels": [c.get("additional_num_kernels") for c in config_dict_list],
+    }
+
+
 def launch_jobs(config_dict_list, input_args, run_eval=True, function_dict=None,
                 require_preload=True):
     """reference: launch_jobs.py:44-122."""
@@ -67,13 +88,12 @@ def launch_jobs(config_dict_list, input_args, run_eval=True, function_dict=None,
     sched_lib = fe.load_scheduler_library()
     py_scheduler = fe.PyScheduler(sched_lib, num_clients)
 
-    model_names = [c["arch"] for c in config_dict_list]
-    model_files = [c["kernel_file"] for c in config_dict_list]
-    additional_model_files = [c.get("additional_kernel_file") for c in config_dict_list]
-    num_kernels = [c["num_kernels"] for c in config_dict_list]
-    num_iters = [c["num_iters"] for c in config_dict_list]
-    train_list = [c["args"]["train"] for c in config_dict_list]
-    additional_num_kernels = [c.get("additional_num_kernels") for c in config_dict_list]
+    lists = job_lists(config_dict_list)
+    model_names, model_files = lists["model_names"], lists["model_files"]
+    additional_model_files = lists["additional_model_files"]
+    num_kernels, num_iters = lists["num_kernels"], lists["num_iters"]
+    train_list = lists["train_list"]
+    additional_num_kernels = lists["additional_num_kernels"]
 
     tids, threads, results = [], [], [None] * num_clients
     for i, config_dict in enumerate(config_dict_list):

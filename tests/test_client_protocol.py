@@ -1,0 +1,162 @@
+"""The Python side of the path: arrival schedules, latency accounting, the
+request loop's barrier protocol, job-file handling, front-end marshalling.
+Pinned by closed forms and by the reference's own job files and arrival trace
+read in place (reference: benchmarking/benchmark_suite/train_imagenet.py:71-241,
+benchmarking/launch_jobs.py:44-148, src/scheduler_frontend.py:17-94)."""
+
+import ctypes
+import glob
+import json
+import os
+import threading
+
+import numpy as np
+import pytest
+
+from orion_amd import launch_jobs
+from orion_amd.benchmark_suite import client_common as cc
+
+
+def test_arrival_gaps_closed_forms():
+    assert cc.arrival_gaps(50, True, 4) == [0.02] * 4
+    assert cc.arrival_gaps(0, False, 3) == [0.0] * 3
+    # the reference seeds numpy's global generator with 42 and then draws
+    # np.random.exponential(scale=1/rps, size=num_iters) (:22-30, :93)
+    np.random.seed(42)
+    want = np.random.exponential(scale=1 / 80, size=100)
+    assert np.array_equal(np.asarray(cc.arrival_gaps(80, False, 100)), want)
+    assert abs(np.mean(cc.arrival_gaps(80, False, 200_000)) - 1 / 80) < 1e-4
+
+
+def test_arrival_trace_file(reference_root, tmp_path):
+    path = os.path.join(reference_root, "artifact_evaluation", "fig10", "inter_arrival_times.json")
+    gaps = cc.arrival_gaps(15, False, 10, input_file=path)
+    assert len(gaps) == 6240
+    assert sum(gaps) == pytest.approx(299.733, abs=1e-3)
+    assert np.mean(gaps) == pytest.approx(0.0480, abs=1e-4)
+
+
+def test_latency_summary_closed_forms():
+    timings = [9.0] * 10 + [i / 1000 for i in range(1, 101)]     # 1..100 ms after warm-up
+    res = cc.latency_summary(timings, batch_idx=110, total_time=2.0, train=False)
+    assert res["p50_latency"] == pytest.approx(50.5)
+    assert res["p95_latency"] == pytest.approx(95.05)
+    assert res["p99_latency"] == pytest.approx(99.01)
+    assert res["throughput"] == pytest.approx((110 - 10) / 2.0)      # :232
+    assert cc.latency_summary(timings, 110, 2.0, train=True) == {"throughput": 50.0}
+    # BERT inference drops 50 requests (bert_trainer_mock.py:213-214)
+    res = cc.latency_summary([9.0] * 50 + [0.002] * 20, 70, 1.0, False, drop=50)
+    assert res["p99_latency"] == pytest.approx(2.0)
+
+
+class FakeBackend:
+    def __init__(self, stop_after=None):
+        self.blocked = []
+        self.stop_after = stop_after
+
+    def block(self, it):
+        self.blocked.append(it)
+
+    def stop(self):
+        return self.stop_after is not None and len(self.blocked) >= self.stop_after
+
+
+class CountingBarrier:
+    def __init__(self):
+        self.waits_at = []
+        self.owner = None
+
+    def wait(self):
+        self.waits_at.append(len(self.owner.blocked))
+
+
+def _run(train, num_iters, rps=0, stop_after=None, tmp_path=None):
+    backend = FakeBackend(stop_after)
+    barrier = CountingBarrier()
+    barrier.owner = backend
+    os.environ["ORION_RESULT_DIR"] = str(tmp_path)
+    steps = []
+    res = cc.run_client(7, train, num_iters, cc.arrival_gaps(rps, True, num_iters), [barrier],
+                        steps.append, backend)
+    return res, steps, backend, barrier
+
+
+def test_request_loop_protocol_training(tmp_path):
+    res, steps, backend, barrier = _run(True, 25, tmp_path=tmp_path)
+    assert steps == list(range(25)) and backend.blocked == list(range(25))
+    # rendezvous after iterations 1 and 10 (:160-165) and once at the end (:217)
+    assert barrier.waits_at == [1, 10, 25]
+    assert res["iterations"] == 25 and "p50_latency" not in res
+    saved = json.load(open(tmp_path / "client_7.json"))
+    assert saved["throughput"] == res["throughput"]
+
+
+def test_request_loop_protocol_inference_and_stop(tmp_path):
+    res, steps, backend, barrier = _run(False, 40, rps=2000, tmp_path=tmp_path)
+    assert steps == list(range(40)) and barrier.waits_at == [1, 10, 40]
+    assert set(res) >= {"p50_latency", "p95_latency", "p99_latency", "throughput"}
+    # open loop: request i is due 1/rps after request i-1, so 30 requests after
+    # warm-up cannot finish faster than 29 gaps
+    assert (40 - 10) / res["throughput"] >= 29 / 2000 * 0.95
+    # a stop request ends the loop after the current iteration (:202-204)
+    res, steps, backend, barrier = _run(True, 1000, stop_after=13, tmp_path=tmp_path)
+    assert len(steps) == 13 and barrier.waits_at == [1, 10, 13]
+
+
+def test_job_lists_accept_the_references_job_files(reference_root):
+    files = [os.path.join(reference_root, "artifact_evaluation", "example", "config.json"),
+             os.path.join(reference_root, "benchmarking", "multi_client_example.json")]
+    files += sorted(glob.glob(os.path.join(reference_root, "artifact_evaluation", "fig7",
+                                           "config_files", "*.json")))
+    assert len(files) > 10
+    known = {"resnet50", "resnet101", "mobilenet_v2", "bert", "transformer"}
+    for path in files:
+        with open(path) as f:
+            job = json.load(f)
+        lists = launch_jobs.job_lists(job)
+        n = len(job)
+        assert all(len(v) == n for v in lists.values())
+        assert set(lists["model_names"]) <= known
+        # training clients come with a first-iteration profile and a steady one
+        for i, entry in enumerate(job):
+            if entry["args"]["train"]:
+                assert lists["additional_model_files"][i] is not None
+                assert lists["additional_num_kernels"][i] > 0
+
+
+def test_job_lists_reject_incomplete_entries():
+    with pytest.raises(KeyError):
+        launch_jobs.job_lists([{"arch": "resnet50", "num_kernels": 1, "num_iters": 1, "args": {}}])
+
+
+def test_cli_matches_the_reference():
+    a = launch_jobs.build_parser().parse_args(
+        ["--algo", "reef", "--config_file", "x.json", "--reef_depth", "12",
+         "--orion_max_be_duration", "160000", "--orion_start_update", "5",
+         "--orion_hp_limit", "30"])
+    assert (a.algo, a.config_file, a.reef_depth, a.orion_max_be_duration,
+            a.orion_start_update, a.orion_hp_limit) == ("reef", "x.json", 12, 160000, 5, 30)
+    d = launch_jobs.build_parser().parse_args(["--algo", "orion", "--config_file", "x"])
+    assert (d.reef_depth, d.orion_max_be_duration, d.orion_start_update, d.orion_hp_limit) == (1, 1, 1, 1)
+
+
+def test_launcher_refuses_to_run_without_the_preloaded_library():
+    with pytest.raises(RuntimeError, match="not preloaded"):
+        launch_jobs.check_preloaded()
+
+
+def test_frontend_rejects_mismatched_lists():
+    from orion_amd import scheduler_frontend as fe
+
+    class Lib:
+        def sched_init(self):
+            return 0
+    py = fe.PyScheduler(Lib(), 2)
+    with pytest.raises(ValueError):
+        py.run_scheduler([threading.Barrier(1)], [1], ["a", "b"], ["f", "g"], [None, None],
+                         [1, 1], [None, None], [1, 1], True, True, False, False, 1, 1, 1,
+                         [False, False])
+    with pytest.raises(NotImplementedError):
+        py.run_scheduler([threading.Barrier(1)], [1, 2], ["a", "b"], ["f", "g"], [None, None],
+                         [1, 1], [None, None], [1, 1], True, False, False, False, 1, 1, 1,
+                         [False, False])
