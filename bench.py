@@ -149,6 +149,8 @@ def main():
     ap.add_argument("--kernels-only", action="store_true",
                     help="only the in-process kernel measurements (for profiler runs: "
                          "starts no child process)")
+    ap.add_argument("--pair-requests", type=int, default=300,
+                    help="measured GEMM requests of the scheduled kernel pair")
     ap.add_argument("--workdir", default="")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -180,6 +182,27 @@ def main():
         out["config"]["records_per_iteration"] = co["num_kernels"]
         out["colocation_wall_s"] = time.time() - t0
         out["policy_replay"] = policy_replay(os.path.join(workdir, "colocated"))
+        # configs[1] through the same hot path: GEMM requests (high priority)
+        # beside the triad loop (best effort), default CU masks; back-to-back
+        # requests (the high-priority client never idle) and Poisson arrivals
+        from orion_amd import kernel_pair as kp_child
+        out["kernel_pair_scheduled"] = {}
+        for label, rps in (("closed_loop", 0), ("poisson_400rps", 400)):
+            pair = kp_child.run_child(small=False, check=True, rps=rps,
+                                      hp_iters=args.pair_requests + 10,
+                                      max_be_duration=args.max_be_duration,
+                                      workdir=os.path.join(workdir, "pair_" + label))
+            out["kernel_pair_scheduled"][label] = {
+                "hp_gemm_ms": {"isolated_p50": pair["hp_isolated"]["p50_latency"],
+                               "isolated_p99": pair["hp_isolated"]["p99_latency"],
+                               "colocated_p50": pair["hp_colocated"]["p50_latency"],
+                               "colocated_p99": pair["hp_colocated"]["p99_latency"]},
+                "hp_p99_ratio": (pair["hp_colocated"]["p99_latency"]
+                                 / pair["hp_isolated"]["p99_latency"]),
+                "be_triad_iters_per_s": {"isolated": pair["be_isolated"]["throughput"],
+                                         "colocated": pair["be_colocated"]["throughput"]},
+                "be_retained": pair["be_retained"],
+                "outputs_match_isolated": pair["outputs_match"]}
 
     import torch
     from orion_amd import kernel_pair as kp

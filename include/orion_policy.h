@@ -44,11 +44,13 @@ int orion_profile_row(const char* path, int row, char* name, size_t name_cap,
 /* CU-mask slot for a best-effort record (no reference counterpart).  masks are
  * ascending CU counts, the last one the whole GPU.  -1 for records that are not
  * kernels (rec_class != 0).  With the high-priority client idle (hp_active ==
- * 0) the whole GPU; with a request in flight the smallest mask holding sm_used,
- * never the whole GPU when a partial mask exists.  algo: 0 orion, 1 reef,
- * 2 sequential (the latter two always use the last slot). */
+ * 0) the whole GPU, or the largest partial mask for a kernel whose profiled
+ * duration alone exceeds the best-effort duration budget (long_kernel != 0);
+ * with a request in flight the smallest mask holding sm_used, never the whole
+ * GPU when a partial mask exists.  algo: 0 orion, 1 reef, 2 sequential (the
+ * latter two always use the last slot). */
 int orion_place_cu_slot(const int* masks, int n_masks, int rec_class,
-                        int sm_used, int algo, int hp_active);
+                        int sm_used, int algo, int hp_active, int long_kernel);
 
 #ifdef __cplusplus
 }

@@ -32,6 +32,8 @@ decision log
     ``T <client>``                                  stop raised for a client
 """
 
+import numpy as np
+
 from oracle import policy_oracle as po
 
 
@@ -46,19 +48,24 @@ class DecisionLog:
         return "\n".join(self.lines) + ("\n" if self.lines else "")
 
 
-def place_cu_slot(masks, cls, sm_used, algo, hp_active):
+def place_cu_slot(masks, cls, sm_used, algo, hp_active, long_kernel=False):
     """CU-mask placement of a best-effort dispatch (no reference counterpart:
     the reference has one stream per client).  ``masks`` is the ascending list
     of mask sizes a best-effort client owns; the last entry is the whole GPU.
-    High-priority client idle: the whole GPU.  Request in flight: the smallest
-    mask that holds the kernel's profiled CU need, never the whole GPU when a
-    partial mask exists.  Records that are not kernels stay where the client's
-    previous op ran (-1)."""
+    High-priority client idle: the whole GPU, unless the kernel alone outlasts
+    the best-effort duration budget (``long_kernel``) -- a request arriving
+    behind it cannot be protected in time, so it is confined to the largest
+    partial mask and leaves the other CUs free.  Request in flight: the
+    smallest mask that holds the kernel's profiled CU need, never the whole
+    GPU when a partial mask exists.  Records that are not kernels stay where
+    the client's previous op ran (-1)."""
     if cls != po.KERNEL:
         return -1
     last = len(masks) - 1
-    if algo != po.ALGO_ORION or not hp_active or last == 0:
+    if algo != po.ALGO_ORION or last == 0:
         return last
+    if not hp_active:
+        return last - 1 if long_kernel else last
     for slot in range(last):
         if sm_used <= masks[slot]:
             return slot
@@ -76,6 +83,7 @@ class RecordingEnv(po.Env):
         self.masks = list(masks)
         self.ops_of = ops_of          # callable(client, op_index) -> OpInfo
         self.algo = algo
+        self.budget = None            # Orion's best-effort duration budget (ns)
         self.obs = []
         self.dec = DecisionLog()
         self._reset_poll()
@@ -150,9 +158,11 @@ class RecordingEnv(po.Env):
         elif owner == self.n - 1:      # the high-priority stream is unmasked
             cu_slot = 0
         else:
-            cu_slot = place_cu_slot(self.masks, cls,
-                                    self.ops_of(client, op_index).sm_used,
-                                    self.algo, self.hp_active())
+            op = self.ops_of(client, op_index)
+            cu_slot = place_cu_slot(
+                self.masks, cls, op.sm_used, self.algo, self.hp_active(),
+                self.budget is not None
+                and float(op.duration) > float(np.float32(self.budget)))
         self._dec.append(f"D {client} {owner} {cls} {op_index} {event_slot} "
                          f"{cu_slot}")
         self.inner.dispatch(client, owner, cls, op_index, event_slot)
@@ -275,6 +285,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
             warmup, witers, algo = bool(int(parts[1])), int(parts[2]), parts[3]
             depth, hp_limit, ustart = int(parts[4]), int(parts[5]), int(parts[6])
             rec.algo = algo
+            rec.budget = depth
             rec.dec.add("S")
             oracle.schedule(rec, warmup, witers, algo, depth, hp_limit, ustart,
                             max_polls=len(polls) + 1)

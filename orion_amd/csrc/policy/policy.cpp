@@ -115,10 +115,11 @@ bool parse_profile(const std::string& path, std::vector<OpInfo>* ops,
 }
 
 int place_cu_slot(const std::vector<int>& masks, int rec_class, int sm_used,
-                  int algo, bool hp_active) {
+                  int algo, bool hp_active, bool long_kernel) {
   if (rec_class != REC_KERNEL) return -1;
   const int last = (int)masks.size() - 1;
-  if (algo != ALGO_ORION || !hp_active || last == 0) return last;
+  if (algo != ALGO_ORION || last == 0) return last;
+  if (!hp_active) return long_kernel ? last - 1 : last;
   for (int s = 0; s < last; ++s)
     if (sm_used <= masks[s]) return s;
   return last - 1;
@@ -170,9 +171,9 @@ void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class) {
   } else if (owner == n_ - 1) {
     d.cu_slot = 0;  // the high-priority stream spans the whole GPU
   } else {
-    d.cu_slot = place_cu_slot(cu_masks_, rec_class,
-                              ops_[client][d.op_index].sm_used, algo_,
-                              seen_[n_ - 1] > 0);
+    const OpInfo& op = ops_[client][d.op_index];
+    d.cu_slot = place_cu_slot(cu_masks_, rec_class, op.sm_used, algo_,
+                              seen_[n_ - 1] > 0, op.duration > (float)be_budget_);
   }
   host.dispatch(d);
   if (rec_class == REC_KERNEL) {
@@ -276,6 +277,7 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
   const bool is_reef = args.algo == ALGO_REEF;
   const bool is_seq = args.algo == ALGO_SEQUENTIAL;
   algo_ = args.algo;
+  be_budget_ = args.depth;
   std::vector<int> profiles(n, -1);
   bool large_found = false;
   long sum = 0;   // outstanding best-effort duration; long += float below

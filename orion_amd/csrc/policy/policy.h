@@ -64,7 +64,7 @@ bool parse_profile(const std::string& path, std::vector<OpInfo>* ops,
 // the high-priority client.  Records that are not kernels stay where the
 // client's work is (-1).
 int place_cu_slot(const std::vector<int>& masks, int rec_class, int sm_used,
-                  int algo, bool hp_active);
+                  int algo, bool hp_active, bool long_kernel);
 
 struct Dispatch {
   int client;      // whose record
@@ -149,6 +149,7 @@ class Policy {
   bool large_found_ = false;
   long sum_ = 0;
   int algo_ = ALGO_ORION;
+  int be_budget_ = 0;  // Orion's best-effort duration budget of this call (ns)
   bool changed_ = false;
 };
 

@@ -75,10 +75,11 @@ int orion_profile_row(const char* path, int row, char* name, size_t name_cap,
 }
 
 int orion_place_cu_slot(const int* masks, int n_masks, int rec_class,
-                        int sm_used, int algo, int hp_active) {
+                        int sm_used, int algo, int hp_active, int long_kernel) {
   std::vector<int> m(masks, masks + (n_masks > 0 ? n_masks : 0));
   if (m.empty()) return -1;
-  return orion::place_cu_slot(m, rec_class, sm_used, algo, hp_active != 0);
+  return orion::place_cu_slot(m, rec_class, sm_used, algo, hp_active != 0,
+                              long_kernel != 0);
 }
 
 }  // extern "C"

@@ -186,7 +186,7 @@ def pair_job(small=False, hp_iters=60, rps=0):
 
 
 def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
-              max_be_duration=1_000_000, algo="orion", reef_depth=12):
+              max_be_duration=1_000_000, algo="orion", reef_depth=12, rps=0):
     """Profile both clients and run the pair isolated and co-located, in child
     processes with the interception library preloaded.  Returns the experiment
     summary (see ``colocate.experiment``) plus ``outputs_match`` when ``check``."""
@@ -196,7 +196,7 @@ def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
     os.makedirs(workdir, exist_ok=True)
     cfg = os.path.join(workdir, "pair.json")
     with open(cfg, "w") as f:
-        json.dump(pair_job(small, hp_iters), f)
+        json.dump(pair_job(small, hp_iters, rps), f)
     filled = os.path.join(workdir, "pair_filled.json")
     env = colocate.preload_env({"ORION_RESULT_DIR": workdir})
     subprocess.run([sys.executable, "-m", "orion_amd.profiling.capture_profile", "--config",

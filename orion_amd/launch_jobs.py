@@ -12,6 +12,7 @@ preloaded, as the reference is (artifact_evaluation/README.md:75)::
 """
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -39,9 +40,11 @@ def _function_dict():
 def check_preloaded():
     """The interception library only sees the clients' HIP calls when the
     dynamic linker put it first; refuse to run a job without it."""
-    with open("/proc/self/maps") as f:
-        loaded = f.read()
-    if "libinttemp.so" not in loaded:
+    # A preloaded library sits in the global symbol scope; one that was only
+    # dlopen()ed later does not, and would not interpose anything either.
+    try:
+        ctypes.CDLL(None).orion_capture_arm
+    except AttributeError:
         raise RuntimeError(
             "libinttemp.so is not preloaded: start the launcher with "
             f"LD_PRELOAD={_lib.CAPTURE_LIB} (append to any value already set)")

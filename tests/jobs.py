@@ -113,6 +113,7 @@ def run_oracle(job, max_polls=3_000_000):
     rec = obslog.RecordingEnv(env, job.n, job.masks,
                               lambda c, k: oracle.ops[c][k], algo=job.algo,
                               hp_active=lambda: oracle.seen[job.n - 1] > 0)
+    rec.budget = job.depth
     rec.header(job.max_sms, [(job.nk[c], job.iters[c], job.train[c],
                               job.paths[c]) for c in range(job.n)])
     changes = {1: [(c, po.parse_profile(path), nk, path)
@@ -147,7 +148,7 @@ def policy_lib():
             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)]
         lib.orion_place_cu_slot.argtypes = [
             ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int,
-            ctypes.c_int, ctypes.c_int, ctypes.c_int]
+            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _policy = lib
     return _policy
 

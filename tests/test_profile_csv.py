@@ -151,15 +151,21 @@ def test_cu_slot_placement_matches_oracle():
         for cls in po.ALL_CLASSES:
             for sm in [0, 1, 32, 33, 64, 65, 128, 129, 256, 257, 12544]:
                 for active in (False, True):
-                    want = obslog.place_cu_slot(masks, cls, sm, algo, active)
-                    got = lib.orion_place_cu_slot(arr, 4, cls_id[cls], sm, algo_id,
-                                                  int(active))
-                    assert got == want
+                    for long_k in (False, True):
+                        want = obslog.place_cu_slot(masks, cls, sm, algo, active, long_k)
+                        got = lib.orion_place_cu_slot(arr, 4, cls_id[cls], sm, algo_id,
+                                                      int(active), int(long_k))
+                        assert got == want
     # hand-worked: idle -> whole GPU; active -> smallest mask that holds the
     # need, capped below the whole GPU; a single mask leaves no choice
     place = obslog.place_cu_slot
     assert place(masks, po.KERNEL, 33, po.ALGO_ORION, False) == 3
     assert place(masks, po.KERNEL, 33, po.ALGO_ORION, True) == 1
+    # a kernel that alone outlasts the duration budget never gets every CU
+    assert place(masks, po.KERNEL, 33, po.ALGO_ORION, False, True) == 2
+    assert place(masks, po.KERNEL, 33, po.ALGO_ORION, True, True) == 1
+    assert place([256], po.KERNEL, 33, po.ALGO_ORION, False, True) == 0
+    assert place(masks, po.KERNEL, 33, po.ALGO_REEF, False, True) == 3
     assert place(masks, po.KERNEL, 4000, po.ALGO_ORION, True) == 2
     assert place(masks, po.KERNEL, 1, po.ALGO_ORION, True) == 0
     assert place(masks, po.MEMCPY, 1, po.ALGO_ORION, True) == -1
