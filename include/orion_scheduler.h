@@ -99,6 +99,10 @@ int stop(void);
 void orion_register_thread(int client);
 void orion_register_stream(void* stream);
 int orion_client_index(void);
+/* The client a call naming `stream` from the calling thread would be queued
+ * for; negative when the call would go straight to the runtime (reference
+ * counterpart of the lookup: get_idx, src/cuda_capture/utils_interc.cpp:3-51). */
+int orion_client_of_stream(void* stream);
 
 /* No reference counterpart: while on, the calling thread's HIP calls bypass the
  * queues.  Client loops use it around model construction and library

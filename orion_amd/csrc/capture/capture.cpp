@@ -262,6 +262,10 @@ void orion_register_stream(void* stream) {
 
 int orion_client_index(void) { return client_for_call(nullptr); }
 
+// The client a call naming `stream` from the calling thread would be queued
+// for, or a negative value when it would go straight to the runtime.
+int orion_client_of_stream(void* stream) { return client_for_call((hipStream_t)stream); }
+
 // While on, the calling thread's HIP calls go straight to the runtime: used by
 // a client for work that must not count as part of an iteration (building the
 // model, library auto-tuning runs whose kernel count is not reproducible).

@@ -20,7 +20,8 @@ def declared(header):
 
 
 CAPTURE_SYMBOLS = {"block", "stop", "orion_register_thread", "orion_register_stream",
-                   "orion_client_index", "orion_thread_passthrough"}
+                   "orion_client_index", "orion_client_of_stream",
+                   "orion_thread_passthrough"}
 
 
 def test_kernels_header():
