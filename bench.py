@@ -206,7 +206,7 @@ def main():
 
     import torch
     from orion_amd import kernel_pair as kp
-    reps = max(5, min(50, args.steps // 60))
+    reps = max(20, min(200, args.steps // 6))
     alone = kp.measure_alone(reps=reps)
     pairs = [kp.measure_pair(m, reps=reps) for m in (32, 64, 128, 0)]
     gemm = alone["gemm"]

@@ -39,7 +39,7 @@ int orion_triad_f32(float* a, const float* b, const float* c, float s,
  * both K-contiguous (row-major A, row-major B = the weight layout of a linear
  * layer).  Accumulation is fp32 on the matrix cores; C is fp32 when
  * out_is_f32 != 0, else bf16 rounded to nearest even.  Requires M % 256 == 0,
- * N % 256 == 0, K % 32 == 0 (ORION_ERR_SHAPE otherwise).
+ * N % 256 == 0, K % 64 == 0 (ORION_ERR_SHAPE otherwise).
  * Compute-bound stand-in for conv_trainer.py:20-27 of the reference. */
 int orion_gemm_bf16_nt(const void* A, const void* B, void* C, int M, int N,
                        int K, int out_is_f32, void* stream);

@@ -3,23 +3,26 @@
 //
 // MFMA-bound: 2*M*N*K flops against (M*K + N*K) * 2 + M*N * sizeof(out)
 // algorithmic bytes.  Both operands are K-contiguous, so one 16-byte load gives
-// a lane the eight consecutive K values v_mfma_f32_32x32x16_bf16 wants.
+// a lane the eight consecutive K values v_mfma_f32_16x16x32_bf16 wants.
 //
 // Tiling (64-wide wavefronts, one workgroup resident per CU):
-//   workgroup  256 x 256 x 32   4 wavefronts, 2 x 2
-//   wavefront  128 x 128        4 x 4 MFMA tiles of 32 x 32, 256 accumulators
-//   LDS        4 stages x (A 16 KiB + B 16 KiB) = 128 KiB of the CU's 160 KiB,
-//              filled straight from global memory (global_load_lds_dwordx4),
-//              two k-tiles ahead of the one being multiplied
-// An LDS row is 64 bytes (four 16-byte chunks).  Two rows form a 128-byte
-// super-row; chunk c of row r sits at position ((r & 1) * 4 + c) ^ ((r >> 1) & 7)
-// of its super-row, so the 16-byte fragment reads of any eight consecutive lanes
-// (eight consecutive rows, same logical chunk) cover all banks exactly once.
+//   workgroup  256 x 256 x 64   4 wavefronts, 2 x 2
+//   wavefront  128 x 128        8 x 8 tiles of v_mfma_f32_16x16x32_bf16, 256
+//                               accumulators; a k-tile is two MFMA k-steps
+//   LDS        2 stages x (A 32 KiB + B 32 KiB) = 128 KiB of the CU's 160 KiB,
+//              filled straight from global memory (global_load_lds_dwordx4)
+// An LDS row is one 128-byte cache line of an operand row (eight 16-byte
+// chunks); chunk c of row r sits at position c ^ (r & 7), so the 16-byte
+// fragment reads of any eight consecutive lanes (eight consecutive rows, same
+// logical chunk) cover all banks exactly once.
 //
-// Issue order inside a k-tile (one wave per SIMD, so nothing else hides a
-// stall): every group of four MFMAs is preceded by the two fragment reads the
-// NEXT k-step needs and followed by one global->LDS load of the tile two ahead;
-// bursts of LDS reads or of loads in front of the MFMAs cost 8-25 % here.
+// What shaped it, measured on MI355X at 8192^3 (the GPU sits at its 1400 W
+// power limit throughout, so speed is energy per flop as much as overlap):
+// v_mfma_f32_16x16x32_bf16 sustains 15 % more than 32x32x16 on random data;
+// loading whole 128-byte lines per row (k-tile 64) instead of half lines took
+// the global->LDS stream alone from 0.64 to 0.44 ms; with one wave per SIMD the
+// matrix core idles whenever the wave issues anything else for longer than one
+// MFMA runs, so every other instruction sits alone between two MFMAs.
 //
 // The reference system has no device code of its own; this kernel stands in for
 // the compute-bound half of its toy co-location pair
@@ -36,20 +39,28 @@ namespace {
 
 constexpr int BM = 256;
 constexpr int BN = 256;
-constexpr int BK = 32;
+constexpr int BK = 64;
 constexpr int kThreads = 256;
-constexpr int kStages = 4;
-constexpr int kMatBytes = BM * BK * 2;      // 16 KiB per operand and stage
+constexpr int kStages = 2;
+constexpr int kMatBytes = BM * BK * 2;      // 32 KiB per operand and stage
 constexpr int kStageBytes = 2 * kMatBytes;  // A then B
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
   uint32_t u = __builtin_bit_cast(uint32_t, f);
   if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
   u += 0x7fffu + ((u >> 16) & 1u);
   return (uint16_t)(u >> 16);
+}
+
+// c += a * b on the matrix core; c lives in accumulator registers and is
+// updated in place (as a builtin call the register allocator shuffles the 256
+// accumulators between register files in every iteration).
+__device__ __forceinline__ void mfma_16x16x32(f32x4& c, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
 __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
@@ -104,8 +115,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_bf16_nt_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform
   const int wm = wave >> 1;
   const int wn = wave & 1;
-  const int lrow = lane & 31;
-  const int lhalf = lane >> 5;
+  const int l16 = lane & 15;  // row (A, B) or column (C) within a 16x16 tile
+  const int lq = lane >> 4;   // 16-byte k chunk of a fragment; row group of C
 
   int tm, tn;
   tile_of_block(blockIdx.x, M / BM, N / BN, &tm, &tn);
@@ -114,122 +125,157 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_bf16_nt_kernel(
 
   // Global -> LDS without a stop in registers: global_load_lds_dwordx4 writes
   // the 16 bytes a lane loads to LDS at (wave-uniform base) + lane * 16, so one
-  // instruction of a wave fills eight super-rows (sixteen rows).  Lane l owns
-  // super-row l / 8, PHYSICAL position l % 8 and fetches the (row, chunk) the
-  // swizzle stores there: v = (l % 8) ^ (l / 8), row = 2 * (l / 8) + v / 4,
-  // chunk = v % 4.  Wave w issues row groups w, w + 4, w + 8, w + 12 of A and B.
-  const int v = (lane & 7) ^ (lane >> 3);
-  const int l_row = wave * 16 + (lane >> 3) * 2 + (v >> 2);
-  const int l_chunk = v & 3;
+  // instruction of a wave fills eight 128-byte rows, each a whole cache line of
+  // the operand.  Lane l owns row l / 8, PHYSICAL chunk l % 8 and fetches the
+  // logical chunk the swizzle stores there, (l % 8) ^ (l / 8).  Wave w issues row
+  // blocks w, w + 4, ..., w + 28 of A and of B.
+  const int l_chunk = (lane & 7) ^ (lane >> 3);
+  const int l_row = wave * 8 + (lane >> 3);
   const uint16_t* gA = A + (row0_a + l_row) * (size_t)K + l_chunk * 8;
   const uint16_t* gB = B + (row0_b + l_row) * (size_t)K + l_chunk * 8;
-  const size_t g_step = (size_t)64 * K;  // 64 rows between a wave's row groups
+  const size_t g_step = (size_t)32 * K;  // 32 rows between a wave's row blocks
 
-  // idx 0..3: row groups of A, 4..7: of B
+  // idx 0..7: row blocks of A, 8..15: of B
   auto load_one = [&](int kt, int stage, int idx) {
-    const int i = idx & 3;
-    const uint16_t* p = (idx < 4 ? gA : gB) + (size_t)kt * BK + i * g_step;
-    unsigned char* d = lds + stage * kStageBytes + (idx < 4 ? 0 : kMatBytes) +
+    const int i = idx & 7;
+    const uint16_t* p = (idx < 8 ? gA : gB) + (size_t)kt * BK + i * g_step;
+    unsigned char* d = lds + stage * kStageBytes + (idx < 8 ? 0 : kMatBytes) +
                        (i * 4 + wave) * 1024;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
                                      (__attribute__((address_space(3))) void*)d, 16, 0, 0);
   };
 
-  f32x16 acc[4][4];
+  f32x4 acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-  // Fragment reads.  Fragment i of a wave covers rows base + i*32 + lrow; base
-  // and i*32 are multiples of 16, so the swizzle terms depend on lrow only.
-  const int fr_sw = (lrow >> 1) & 7;
-  const int fr_sub4 = (lrow & 1) * 4;
-  const int fr_a = ((wm * 128 + lrow) >> 1) * 128;
-  const int fr_b = ((wn * 128 + lrow) >> 1) * 128;
-  // Two fragment register sets: the MFMAs of one k-step run out of one set
-  // while the reads of the next k-step fill the other.
-  bf16x8 fa[2][4], fb[2][4];
-  auto read_one = [&](int set, int stage, int kk, int i) {
-    const unsigned char* sa = lds + stage * kStageBytes + fr_a;
-    const unsigned char* sb = lds + stage * kStageBytes + kMatBytes + fr_b;
-    const int off = ((fr_sub4 + kk * 2 + lhalf) ^ fr_sw) << 4;
-    fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + i * 16 * 128 + off);
-    fb[set][i] = *reinterpret_cast<const bf16x8*>(sb + i * 16 * 128 + off);
+  // Fragment reads.  Fragment i of a wave covers rows base + i*16 + l16; of each
+  // 128-byte row, k-step ks uses logical chunks ks*4 .. ks*4+3 and lane group lq
+  // takes chunk ks*4 + lq.  base and i*16 are multiples of 8, so the swizzle term
+  // is l16 % 8.
+  const int fr_a = (wm * 128 + l16) * 128;
+  const int fr_b = kMatBytes + (wn * 128 + l16) * 128;
+  const int fr_k0 = (lq ^ (l16 & 7)) << 4;
+  const int fr_k1 = ((4 + lq) ^ (l16 & 7)) << 4;
+  // Two fragment register sets, one per k-step of a tile.
+  bf16x8 fa[2][8], fb[2][8];
+  auto read_one = [&](auto ks_c, int stage, int r) {
+    constexpr int KS = decltype(ks_c)::value;
+    const unsigned char* st = lds + stage * kStageBytes + (KS ? fr_k1 : fr_k0);
+    if (r < 8) fb[KS][r] = *reinterpret_cast<const bf16x8*>(st + fr_b + r * 2048);
+    else fa[KS][r - 8] = *reinterpret_cast<const bf16x8*>(st + fr_a + (r - 8) * 2048);
   };
+  using KS0 = std::integral_constant<int, 0>;
+  using KS1 = std::integral_constant<int, 1>;
 
   const int KT = K / BK;
 #pragma unroll
-  for (int idx = 0; idx < 8; ++idx) load_one(0, 0, idx);
+  for (int idx = 0; idx < 16; ++idx) load_one(0, 0, idx);
   if (KT > 1) {
 #pragma unroll
-    for (int idx = 0; idx < 8; ++idx) load_one(1, 1, idx);
+    for (int idx = 0; idx < 16; ++idx) load_one(1, 1, idx);
+    __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16): tile 0 has landed
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
   }
-  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) read_one(0, 0, 0, i);
+  for (int r = 0; r < 16; ++r) read_one(KS0{}, 0, r);
 
-  // One k-tile.  Invariant on entry: LDS stage kt % 4 holds tile kt, fragment
-  // set 0 holds its first k-step, every load of tile kt + 1 has been issued.
-  // The barrier sits between the two k-steps: the second step's MFMAs cover it
-  // and the first fragment reads of tile kt + 1.  Tile kt + 2 is loaded into the
-  // stage that held tile kt - 2, whose last read lies before the previous
-  // iteration's barrier.
-  auto k_tile = [&](int kt, auto with_loads) {
-    constexpr bool kLoads = decltype(with_loads)::value;
-    const int cur = kt & 3, nxt = (kt + 1) & 3, ld = (kt + 2) & 3;
+  // One k-tile = two MFMA k-steps of 64 MFMAs.  With one wave per SIMD the
+  // matrix core idles whenever the wave issues anything else for longer than one
+  // MFMA runs (16 cycles), so every other instruction sits alone between two
+  // MFMAs: a fragment read after every third MFMA (all sixteen are out by the
+  // 47th, the last sixteen MFMAs cover their latency), a global->LDS load after
+  // every fourth in the second k-step.
+  //
+  // On entry set 0 holds the first k-step of tile kt and every load of tile
+  // kt + 1 has been issued.  First k-step: fragment reads of the second.  The
+  // wait + barrier after it mean that every wave has all of tile kt in
+  // registers and that tile kt + 1 has landed.  Second k-step: first fragment
+  // reads of tile kt + 1, loads of tile kt + 2 into the stage tile kt has left.
+  auto read_slot = [&](auto ks_c, int stage, int m) {
+    // B fragments first: every MFMA row of the next k-step needs all of them
+    if (m % 3 == 1) read_one(ks_c, stage, m / 3);
+  };
+  auto k_tile = [&](int kt, auto has_next, auto has_loads) {
+    constexpr bool kNext = decltype(has_next)::value;
+    constexpr bool kLoads = decltype(has_loads)::value;
+    const int cur = kt & 1, nxt = cur ^ 1;
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): set 0 is complete
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      read_one(1, cur, 1, i);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
-      if (kLoads) load_one(kt + 2, ld, i);
+    for (int m = 0; m < 64; ++m) {
+      mfma_16x16x32(acc[m >> 3][m & 7], fa[0][m >> 3], fb[0][m & 7]);
+      read_slot(KS1{}, cur, m);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kt + 1 < KT) {
-      // lgkmcnt(0): this wave's reads of stage cur have returned (the stage is
-      // overwritten two iterations on); vmcnt: all but the loads just issued,
-      // i.e. tile kt + 1 has landed.
-      if (kLoads) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
-      else __builtin_amdgcn_s_waitcnt(0x0070);         // vmcnt(0) lgkmcnt(0)
-      __builtin_amdgcn_s_barrier();
-    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    if (kNext) __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (kt + 1 < KT) read_one(0, nxt, 0, i);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
-      if (kLoads) load_one(kt + 2, ld, 4 + i);
+    for (int m = 0; m < 64; ++m) {
+      mfma_16x16x32(acc[m >> 3][m & 7], fa[1][m >> 3], fb[1][m & 7]);
+      if (kNext) read_slot(KS0{}, nxt, m);
+      if (kLoads && (m & 3) == 2) load_one(kt + 2, cur, m >> 2);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   int kt = 0;
-  for (; kt + 2 < KT; ++kt) k_tile(kt, std::true_type{});
-  for (; kt < KT; ++kt) k_tile(kt, std::false_type{});
+  for (; kt + 2 < KT; ++kt) k_tile(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < KT) { k_tile(kt, std::true_type{}, std::false_type{}); ++kt; }
+  k_tile(kt, std::false_type{}, std::false_type{});
 
-  // Epilogue.  Accumulator register r of a 32x32 tile holds
-  // row (r/4)*8 + lhalf*4 + r%4, column lrow.
-  const size_t c_row0 = row0_a + wm * 128;
-  const size_t c_col0 = row0_b + wn * 128 + lrow;
+  // The MFMAs above are opaque to the compiler's hazard handling: give the last
+  // ones time to write their accumulators before anything reads them.
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+  // Epilogue.  Accumulator register r of a 16x16 tile holds row lq*4 + r,
+  // column l16: stored as it lies, a lane would write two bytes at a time in
+  // 32-byte runs.  Each wave instead turns its 128 x 128 block round in its own
+  // quarter of the LDS (free now) and writes whole rows, 16 bytes per lane, so
+  // every store instruction covers full cache lines.  A row is cut into eight
+  // chunks of 16 elements; chunk j of row R sits at position j ^ ((R >> 2) & 3),
+  // which spreads the four row groups of one write over all banks.
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_s_barrier();  // every wave has read its last fragments
+  constexpr int kElt = (int)sizeof(OutT);
+  constexpr int kRowB = 128 * kElt;          // bytes of one row of the block
+  constexpr int kChunkB = 16 * kElt;
+  constexpr int kPassRows = 32768 / kRowB;   // rows that fit the wave's quarter
+  constexpr int kPasses = 128 / kPassRows;   // 1 (bf16) or 2 (fp32)
+  constexpr int kIPerPass = 8 / kPasses;
+  constexpr int kUnits = kRowB / 16;         // 16-byte units per row
+  constexpr int kRowsPerStore = 64 / kUnits;
+  unsigned char* ep = lds + wave * 32768;
+  const int st_row = lane / kUnits;
+  const int st_unit = lane % kUnits;
+  OutT* c_block = C + (row0_a + wm * 128) * (size_t)N + row0_b + wn * 128;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int ii = 0; ii < kIPerPass; ++ii)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const size_t row = c_row0 + i * 32 + (r >> 2) * 8 + lhalf * 4 + (r & 3);
-        const size_t col = c_col0 + j * 32;
-        store_out(C + row * (size_t)N + col, acc[i][j][r]);
-      }
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          store_out(reinterpret_cast<OutT*>(ep + (ii * 16 + lq * 4 + r) * kRowB +
+                                            (j ^ lq) * kChunkB) + l16,
+                    acc[pass * kIPerPass + ii][j][r]);
+#pragma unroll
+    for (int it = 0; it < kPassRows / kRowsPerStore; ++it) {
+      const int R = it * kRowsPerStore + st_row;
+      const int byte = st_unit * 16;
+      const int phys = ((byte / kChunkB) ^ ((R >> 2) & 3)) * kChunkB + byte % kChunkB;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(ep + R * kRowB + phys);
+      __builtin_nontemporal_store(
+          v, reinterpret_cast<u32x4*>(c_block + (size_t)(pass * kPassRows + R) * N) + st_unit);
+    }
+  }
 }
 
 }  // namespace

@@ -90,7 +90,7 @@ def _gemm_case(m, n, k, seed):
     return a, b, ta, tb
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 32), (256, 256, 64), (256, 256, 96), (256, 512, 128), (512, 256, 1024),
+@pytest.mark.parametrize("shape", [(256, 256, 64), (256, 256, 128), (256, 256, 192), (256, 512, 256), (512, 256, 1024),
                                    (768, 1024, 512), (1024, 1024, 2048)])
 def test_gemm_against_exact_product(shape):
     m, n, k = shape
@@ -139,11 +139,12 @@ def test_gemm_full_size_sampled_rows_and_identity():
 
 
 def test_gemm_rejects_bad_shapes_without_launching():
-    a = torch.zeros(256, 80, device=DEV, dtype=torch.bfloat16)
-    b = torch.zeros(256, 80, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(kernels.KernelError) as e:
-        kernels.gemm_bf16_nt(a, b)                    # K not a multiple of 32
-    assert e.value.code == 2
+    for k in (80, 96):                                # K not a multiple of 64
+        a = torch.zeros(256, k, device=DEV, dtype=torch.bfloat16)
+        b = torch.zeros(256, k, device=DEV, dtype=torch.bfloat16)
+        with pytest.raises(kernels.KernelError) as e:
+            kernels.gemm_bf16_nt(a, b)
+        assert e.value.code == 2
     a = torch.zeros(100, 64, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(kernels.KernelError) as e:
         kernels.gemm_bf16_nt(a, torch.zeros(256, 64, device=DEV, dtype=torch.bfloat16))
