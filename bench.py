@@ -58,9 +58,6 @@ def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False):
     cfg = os.path.join(workdir, "job.json")
     with open(cfg, "w") as f:
         json.dump(c3_job(steps + 10), f)
-    # children inherit the preload through the environment
-    os.environ.update({k: v for k, v in colocate.preload_env().items()
-                       if k == "LD_PRELOAD"})
     job = capture_profile.fill_job(cfg, os.path.join(workdir, "profiles"),
                                    os.path.join(workdir, "job_filled.json"), quiet=True,
                                    use_rocprof=use_rocprof)
@@ -71,9 +68,6 @@ def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False):
     res = colocate.experiment(job, "orion", max_be_duration, workdir, env=env)
     res["num_kernels"] = {"hp": job[-1]["num_kernels"],
                           "be": job[0].get("additional_num_kernels", job[0]["num_kernels"])}
-    os.environ["LD_PRELOAD"] = ":".join(
-        p for p in os.environ.get("LD_PRELOAD", "").split(":")
-        if p and "libinttemp.so" not in p)
     return res
 
 

@@ -117,7 +117,7 @@ CaptureState* orion_capture_state(void) { return &g_state; }
 
 // Status a record carries when the scheduler hands a blocking call back to the
 // thread that made it.
-enum { ORION_GRANTED_TO_CALLER = -1000 };
+enum { ORION_GRANTED_TO_CALLER = orion::kRecordGranted };
 
 bool orion_record_runs_on_caller(int type) {
   return type == RT_MALLOC || type == RT_FREE || type == RT_MEMCPY ||
@@ -219,6 +219,7 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
     ch.stop.store(0);
     ch.stop_ack.store(0);
     ch.last_stream.store(nullptr);
+    ch.direct_stream.store(nullptr);
     ch.submitted.store(0);
     ch.block_calls.store(0);
     // own_streams survive: a client may register its stream before setup runs
@@ -317,6 +318,26 @@ int submit(int idx, Record& r, bool wait) {
   Record* slot = &ch.slots[ticket & (kQueueSlots - 1)];
   r.status = 0;
   r.sync_stream = nullptr;
+  if (hipStream_t direct = ch.direct_stream.load(std::memory_order_acquire)) {
+    // The scheduler lets this client issue its own calls: run the call here, on
+    // the stream the scheduler named, under the producer lock so that the
+    // notices reach the queue in issue order; nobody waits for the notice.
+    int st;
+    if (orion_record_runs_on_caller(r.type)) {
+      st = execute_on_caller(r, direct);
+    } else {
+      ++tl_bypass;
+      st = orion_execute_record(&r, direct);
+      --tl_bypass;
+    }
+    ch.last_stream.store(direct, std::memory_order_release);
+    r.status = kRecordIssued;
+    *slot = r;
+    ch.tail.store(ticket + 1, std::memory_order_release);
+    ch.submitted.fetch_add(1, std::memory_order_relaxed);
+    ch.producer_lock.store(0, std::memory_order_release);
+    return st;
+  }
   *slot = r;
   ch.tail.store(ticket + 1, std::memory_order_release);
   ch.submitted.fetch_add(1, std::memory_order_relaxed);

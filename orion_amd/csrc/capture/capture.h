@@ -116,6 +116,10 @@ struct Record {
   } u;
 };
 
+// Record::status values outside the HIP error range.
+constexpr int32_t kRecordGranted = -1000;  // scheduler -> caller: run it yourself
+constexpr int32_t kRecordIssued = -1001;   // caller -> scheduler: already issued
+
 constexpr int kMaxClients = 32;
 constexpr uint32_t kQueueSlots = 8;   // power of two; occupancy is <= 2 in practice
 
@@ -135,6 +139,12 @@ struct alignas(64) ClientChannel {
   // streams the client itself names (its torch stream), for calls made on its
   // behalf by threads that are not registered (autograd workers)
   std::atomic<hipStream_t> own_streams[4];
+  // Non-null while the scheduler lets this client issue its own calls: the
+  // client executes each call on this stream at once and queues the record only
+  // as a notice (status kRecordIssued), without waiting for it to be retired.
+  // Used for a high-priority inference client, whose records the policy
+  // dispatches unconditionally in the poll it sees them.
+  std::atomic<hipStream_t> direct_stream;
   std::atomic<uint64_t> submitted;      // records pushed, all types
   std::atomic<int64_t> block_calls;     // highest it+1 the client passed to block()
 };

@@ -30,7 +30,7 @@ bool orion_record_runs_on_caller(int type);
 namespace {
 
 using namespace orion;
-constexpr int kGrantedToCaller = -1000;
+constexpr int kGrantedToCaller = orion::kRecordGranted;
 
 struct Row {
   int iteration, index, type;

@@ -52,7 +52,7 @@ namespace {
 using namespace orion;
 using Clock = std::chrono::steady_clock;
 
-constexpr int kGrantedToCaller = -1000;  // keep equal to capture.cpp
+constexpr int kGrantedToCaller = orion::kRecordGranted;
 
 [[noreturn]] void die(const std::string& what) {
   fprintf(stderr, "orion scheduler: %s\n", what.c_str());
@@ -120,6 +120,12 @@ class LiveHost : public PolicyHost {
     update_owner_ = owner;
     update_slot_ = slot;
     update_valid_ = false;
+  }
+  // Lets `client` issue its own calls on its widest stream (see
+  // ClientChannel::direct_stream), or takes that permission back.
+  void set_direct(int client, bool on) {
+    hipStream_t s = on ? streams_[(size_t)client].back() : nullptr;
+    cap_->channels[client].direct_stream.store(s, std::memory_order_release);
   }
   void begin_phase() {
     last_progress_ = Clock::now();
@@ -209,7 +215,9 @@ class LiveHost : public PolicyHost {
     cur_cu_slot_[(size_t)d.client] = slot;
     ch.last_stream.store(stream, std::memory_order_release);
 
-    if (orion_record_runs_on_caller(rec->type)) {
+    if (rec->status == orion::kRecordIssued) {
+      // the client has issued this call itself, on the stream set_direct gave it
+    } else if (orion_record_runs_on_caller(rec->type)) {
       rec->sync_stream = stream;
       rec->status = kGrantedToCaller;
     } else {
@@ -352,6 +360,7 @@ struct Global {
   std::vector<bool> is_train;
   std::string record_dir;
   bool verbose = true;
+  bool hp_direct = true;  // ORION_HP_DIRECT=0: every client hands every call over
 };
 Global g;
 int g_handle_token = 0;
@@ -395,6 +404,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
       die("ORION_BE_CU_MASKS must be an ascending list of positive CU counts");
   if (g.masks.back() < cus) g.masks.push_back(cus);
   if (const char* e = getenv("ORION_QUIET")) g.verbose = atoi(e) == 0;
+  if (const char* e = getenv("ORION_HP_DIRECT")) g.hp_direct = atoi(e) != 0;
 
   std::vector<std::vector<OpInfo>> profiles((size_t)num_clients);
   std::vector<int> nk, ni;
@@ -466,6 +476,13 @@ void* schedule(void* /*scheduler*/, int num_clients, bool profile_mode, int /*it
     g.host->set_update_slot(hp, update_start - 1);
   else
     g.host->set_update_slot(-1, -1);
+  // A high-priority inference client is dispatched unconditionally in the poll
+  // that sees its record (scheduler_eval.cpp:311-321): the decision needs no
+  // wait, so the client issues its calls itself and the queue carries notices.
+  // Not under time slicing (the client must wait its turn) and not for a
+  // training client (the update-phase event must follow one exact kernel).
+  const bool direct = g.hp_direct && a.algo != ALGO_SEQUENTIAL && !g.is_train[(size_t)hp];
+  g.host->set_direct(hp, direct);
   g.host->begin_phase();
   PolicyHost* host = g.host.get();
   if (g.recorder) {
@@ -474,6 +491,7 @@ void* schedule(void* /*scheduler*/, int num_clients, bool profile_mode, int /*it
     host = g.recorder.get();
   }
   g.policy->schedule(*host, a);
+  g.host->set_direct(hp, false);
   if (g.recorder) {
     g.recorder->end_schedule();
     flush_recording();

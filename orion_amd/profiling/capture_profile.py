@@ -137,9 +137,16 @@ def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False, use_rocpr
     additional_* pair) filled in."""
     import subprocess
     import sys
+    from .. import _lib
     with open(config_path) as f:
         job = json.load(f)
     os.makedirs(out_dir, exist_ok=True)
+    # the profiling children need the interception library preloaded; the caller
+    # does not
+    env = dict(os.environ)
+    preload = [p for p in env.get("LD_PRELOAD", "").split(":") if p]
+    if _lib.CAPTURE_LIB not in preload:
+        env["LD_PRELOAD"] = ":".join(preload + [_lib.CAPTURE_LIB])
     done = {}
     for idx, entry in enumerate(job):
         prefix = os.path.abspath(os.path.join(out_dir, profile_name(entry)))
@@ -149,9 +156,9 @@ def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False, use_rocpr
                    "--iters", str(iters)]
             if quiet:     # keep the caller's stdout clean; the log stays beside the profile
                 with open(prefix + ".log", "w") as log:
-                    subprocess.run(cmd, check=True, stdout=log, stderr=subprocess.STDOUT)
+                    subprocess.run(cmd, check=True, stdout=log, stderr=subprocess.STDOUT, env=env)
             else:
-                subprocess.run(cmd, check=True)
+                subprocess.run(cmd, check=True, env=env)
             with open(prefix + ".json") as f:
                 done[prefix] = json.load(f)
             if use_rocprof:

@@ -160,6 +160,10 @@ print(json.dumps({
     "alive": alive, "iters_done": iters_done, "outputs_equal": ok_outputs,
     "launch_tids": launch_tids, "sched_tid": sched_tid, "client_tids": tids,
     "launch_stream_masks": masks, "n_launches": sum(1 for k, s, t in log if k == 0),
+    "launch_streams_by_tid": {str(t): sorted({s for k, s, tt in log if k == 0 and tt == t})
+                              for t in launch_tids},
+    "launches_by_tid": {str(t): sum(1 for k, s, tt in log if k == 0 and tt == t)
+                        for t in launch_tids},
 }))
 sys.stdout.flush()
 os._exit(0 if not any(alive) else 3)

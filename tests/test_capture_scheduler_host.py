@@ -7,7 +7,10 @@ scheduler thread runs the three-phase schedule.  Checked here:
 
 * every client's final buffer equals the same kernel sequence run in isolation
   (bit-exact: the kernels are deterministic host functions);
-* every launch was issued by the scheduler thread, none by a client thread;
+* every launch was issued by the scheduler thread, none by a client thread --
+  except that a high-priority inference client, whose records the policy
+  dispatches unconditionally, issues its own calls on the one unmasked stream
+  the scheduler gave it (ORION_HP_DIRECT=0 switches that off);
 * best-effort kernels ran on CU-masked streams, the high-priority client on an
   unmasked one;
 * the stop protocol ended the best-effort clients once the high-priority client
@@ -30,28 +33,40 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FAKEHIP = os.path.join(ROOT, "tests", "fakehip", "libfakehip.so")
 
 
-def run_child(workdir, algo, n_be, hp_iters):
+def run_child(workdir, algo, n_be, hp_iters, direct=True):
     if not os.path.exists(FAKEHIP):
         pytest.fail("tests/fakehip/libfakehip.so is not built (make -C orion_amd/csrc)")
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), workdir,
          algo, str(n_be), str(hp_iters)],
-        capture_output=True, text=True, timeout=300)
+        capture_output=True, text=True, timeout=300,
+        env=dict(os.environ, ORION_HP_DIRECT="1" if direct else "0"))
     assert proc.returncode == 0, proc.stdout + proc.stderr
     line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
     return json.loads(line)
 
 
+@pytest.mark.parametrize("direct", [True, False])
 @pytest.mark.parametrize("algo,n_be", [("orion", 0), ("orion", 1), ("orion", 3),
                                        ("reef", 2), ("sequential", 1)])
-def test_job_protocol_on_fake_runtime(tmp_path, algo, n_be):
+def test_job_protocol_on_fake_runtime(tmp_path, algo, n_be, direct):
     hp_iters = 40
-    res = run_child(str(tmp_path), algo, n_be, hp_iters)
+    res = run_child(str(tmp_path), algo, n_be, hp_iters, direct)
     assert not any(res["alive"])
     assert res["iters_done"][-1] == hp_iters
     assert all(res["outputs_equal"]), res
-    assert res["launch_tids"] == res["sched_tid"]
-    assert not set(res["launch_tids"]) & set(res["client_tids"])
+    sched, hp_tid = res["sched_tid"][0], res["client_tids"][-1]
+    if direct and algo != "sequential":
+        assert set(res["launch_tids"]) <= {sched, hp_tid}
+        # all but the records queued before the scheduler's first call
+        assert res["launches_by_tid"][str(hp_tid)] >= (hp_iters - 1) * 5
+        hp_streams = res["launch_streams_by_tid"][str(hp_tid)]
+        assert len(hp_streams) == 1 and res["launch_stream_masks"][str(hp_streams[0])] == 0
+        if n_be:
+            assert str(sched) in res["launches_by_tid"]
+    else:
+        assert res["launch_tids"] == res["sched_tid"]
+        assert not set(res["launch_tids"]) & set(res["client_tids"])
     if algo == "orion" and n_be > 0:
         masked = [b for b in res["launch_stream_masks"].values() if b > 0]
         assert masked and all(b in (32, 64, 128) for b in masked)

@@ -38,8 +38,11 @@ def test_capture_and_scheduler_are_race_free(tmp_path):
     env = dict(os.environ, ORION_HIP_LIBRARY=fake, ORION_QUIET="1",
                TSAN_OPTIONS="halt_on_error=1 exitcode=66 second_deadlock_stack=1")
     env.pop("LD_PRELOAD", None)
-    for clients in (2, 4):
-        proc = subprocess.run([exe, str(tmp_path), str(clients), "40"], env=env,
+    # both hand-offs of the high-priority client: issuing its own calls and
+    # queueing notices (default), and the synchronous hand-off of every record
+    for clients, direct in ((2, "1"), (4, "1"), (3, "0")):
+        proc = subprocess.run([exe, str(tmp_path), str(clients), "40"],
+                              env=dict(env, ORION_HP_DIRECT=direct),
                               capture_output=True, text=True, timeout=600)
         assert "WARNING: ThreadSanitizer" not in proc.stderr, proc.stderr[-4000:]
         assert proc.returncode == 0, proc.stdout + proc.stderr[-4000:]
