@@ -85,14 +85,8 @@ def test_resnet50_colocation_outputs_and_replay(tmp_path):
     cfg = os.path.join(work, "job.json")
     with open(cfg, "w") as f:
         json.dump(job, f)
-    env = colocate.preload_env()
-    os.environ["LD_PRELOAD"] = env["LD_PRELOAD"]
-    try:
-        filled = capture_profile.fill_job(cfg, os.path.join(work, "profiles"),
-                                          os.path.join(work, "filled.json"))
-    finally:
-        os.environ["LD_PRELOAD"] = ":".join(
-            p for p in env["LD_PRELOAD"].split(":") if "libinttemp.so" not in p)
+    filled = capture_profile.fill_job(cfg, os.path.join(work, "profiles"),
+                                      os.path.join(work, "filled.json"), quiet=True)
     iso_dir, co_dir = os.path.join(work, "iso_out"), os.path.join(work, "co_out")
     os.makedirs(iso_dir)
     os.makedirs(co_dir)
@@ -121,3 +115,103 @@ def test_resnet50_colocation_outputs_and_replay(tmp_path):
     err = (co_out - ref).abs().max() / ref.abs().max()
     assert err <= CPU_RTOL, float(err)
     _check_replay(co_dir)
+
+
+def _run_iso_and_co(work, job, budget=160000):
+    """Profiles the job's clients, runs the high-priority client alone and the
+    whole job, both saving outputs; returns (filled job, co-located results,
+    isolated HP output, co-located HP output, record dir)."""
+    from orion_amd import colocate
+    from orion_amd.profiling import capture_profile
+    cfg = os.path.join(work, "job.json")
+    with open(cfg, "w") as f:
+        json.dump(job, f)
+    filled = capture_profile.fill_job(cfg, os.path.join(work, "profiles"),
+                                      os.path.join(work, "filled.json"), quiet=True)
+    iso_dir, co_dir = os.path.join(work, "iso_out"), os.path.join(work, "co_out")
+    os.makedirs(iso_dir)
+    os.makedirs(co_dir)
+    colocate.run_job([copy.deepcopy(filled[-1])], "orion", os.path.join(work, "iso"),
+                     budget, env={"ORION_SAVE_OUTPUT_DIR": iso_dir})
+    co = colocate.run_job(copy.deepcopy(filled), "orion", os.path.join(work, "co"),
+                          budget, env={"ORION_SAVE_OUTPUT_DIR": co_dir,
+                                       "ORION_RECORD_DIR": co_dir})
+    hp = len(job) - 1
+    iso_out = torch.load(os.path.join(iso_dir, "client_0_output.pt"), weights_only=True)
+    co_out = torch.load(os.path.join(co_dir, f"client_{hp}_output.pt"), weights_only=True)
+    return filled, co, iso_out, co_out, co_dir
+
+
+def _mobilenet_cpu_reference(batch):
+    from orion_amd.benchmark_suite import client_common as cc
+    from orion_amd.benchmark_suite.train_imagenet import DummyDataLoader
+    from orion_amd.benchmark_suite.vision_models import mobilenet_v2
+    with cc.MODEL_INIT_LOCK:
+        cc.seed_everything(42)
+        model = mobilenet_v2().eval()
+    data, _ = next(DummyDataLoader(batch, 42))
+    with torch.no_grad():
+        return model(data.float())
+
+
+def test_mobilenet_beside_bert_training(tmp_path):
+    """The shape of the reference's MobileNetV2-inference + BERT-training pair
+    (artifact_evaluation/fig7/config_files/bert_mnet.json): a transformer
+    trainer (hipBLASLt / rocBLAS GEMMs, fused attention, AdamW) as the
+    best-effort client."""
+    job = [
+        {"arch": "bert", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"batchsize": 2, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": True, "dtype": "fp32"}},
+        {"arch": "mobilenet_v2", "kernel_file": "", "num_kernels": 0, "num_iters": 40,
+         "args": {"model_name": "mobilenet_v2", "batchsize": 4, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": False, "dtype": "fp32"}},
+    ]
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job, 100000)
+    assert co[-1]["iterations"] == 40 and co[0]["iterations"] >= 10
+    assert filled[0]["num_kernels"] > 500        # a BERT-base training step
+    ref = _mobilenet_cpu_reference(4)
+    for out in (iso_out, co_out):
+        assert float((out - ref).abs().max() / ref.abs().max()) <= CPU_RTOL
+    # depthwise convolutions may take an atomics-based solver: iso and co-located
+    # agree to the same tolerance, not necessarily to the bit
+    assert float((iso_out - co_out).abs().max() / ref.abs().max()) <= CPU_RTOL
+    _check_replay(co_dir)
+
+
+def test_four_clients_round_robin(tmp_path):
+    """N = 4 (reference: multi_client_example.json; round-robin over the
+    best-effort clients, scheduler_eval.cpp:323-326): a model client with three
+    best-effort clients of different kinds."""
+    from orion_amd import kernel_pair
+    job = [
+        {"arch": "triad_f32", "kernel_file": "", "num_kernels": 0, "num_iters": 1_000_000,
+         "args": {"batchsize": 1 << 22, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": True}},
+        {"arch": "gemm_bf16", "kernel_file": "", "num_kernels": 0, "num_iters": 1_000_000,
+         "args": {"batchsize": 1024, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": True}},
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": True}},
+        {"arch": "mobilenet_v2", "kernel_file": "", "num_kernels": 0, "num_iters": 60,
+         "args": {"model_name": "mobilenet_v2", "batchsize": 4, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": False, "dtype": "fp32"}},
+    ]
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job)
+    assert co[-1]["iterations"] == 60
+    assert all(c["iterations"] >= 10 for c in co[:-1])
+    ref = _mobilenet_cpu_reference(4)
+    assert float((co_out - ref).abs().max() / ref.abs().max()) <= CPU_RTOL
+    assert float((iso_out - co_out).abs().max() / ref.abs().max()) <= CPU_RTOL
+    dec = _check_replay(co_dir)
+    # every best-effort client was dispatched after warm-up, in rotation
+    owners = [l.split()[1] for l in dec.splitlines() if l.startswith("D ")]
+    assert {"0", "1", "2", "3"} <= set(owners)
+    # the triad client's result is exact
+    out = torch.load(os.path.join(co_dir, "client_0_output.pt"), weights_only=True)
+    b, c = kernel_pair._inputs_triad(1 << 22, "cuda:0")
+    want = torch.addcmul(b[:4096].double(), c[:4096].double(),
+                         torch.tensor(float(torch.tensor(1.7, dtype=torch.float32)),
+                                      dtype=torch.float64, device="cuda:0")).float().cpu()
+    assert torch.equal(out, want)
