@@ -3,6 +3,14 @@
 // system HIP runtime only, so a profiler sees exactly these kernels.
 //
 //   bench_kernels [--reps N] [--warmup N] [--gemm-n N] [--triad-elems N] [--mask CUS]
+//                 [--pair 1]
+//
+// --pair 1 runs the two kernels at the same time instead: the GEMM on a stream
+// over the whole GPU, the triad on a stream over --mask CUs, submissions
+// interleaved so that neither queue runs dry (a pilot run finds how many triads
+// one GEMM needs).  A kernel trace of that run gives each kernel's duration
+// next to the other; hardware counters cannot, because the profiler serialises
+// dispatches while it collects them.
 //
 // Per kernel it prints the average launch duration measured with HIP events on
 // the stream the kernel runs on, and the achieved rate against its roofline.
@@ -92,8 +100,33 @@ static void launch_copy(hipStream_t s, void* p) {
                      (const f32x4*)t->b, t->n / 4);
 }
 
+// Both kernels at once; returns average ms per launch of each.
+static void run_pair(hipStream_t sg, hipStream_t st, GemmCtx* g, TriadCtx* t, int n_gemm,
+                     int n_triad, float* gemm_ms, float* triad_ms) {
+  hipEvent_t e[4];
+  for (auto& x : e) CHECK(hipEventCreate(&x));
+  for (int i = 0; i < 3; ++i) launch_triad(st, t);  // the other stream is busy first
+  CHECK(hipEventRecord(e[0], sg));
+  CHECK(hipEventRecord(e[2], st));
+  int done_t = 0;
+  for (int i = 0; i < n_gemm; ++i) {
+    launch_gemm(sg, g);
+    const int want = (int)((long long)(i + 1) * n_triad / n_gemm);
+    for (; done_t < want; ++done_t) launch_triad(st, t);
+  }
+  CHECK(hipEventRecord(e[1], sg));
+  CHECK(hipEventRecord(e[3], st));
+  CHECK(hipEventSynchronize(e[1]));
+  CHECK(hipEventSynchronize(e[3]));
+  CHECK(hipEventElapsedTime(gemm_ms, e[0], e[1]));
+  CHECK(hipEventElapsedTime(triad_ms, e[2], e[3]));
+  *gemm_ms /= n_gemm;
+  *triad_ms /= (done_t > 0 ? done_t : 1);
+  for (auto& x : e) CHECK(hipEventDestroy(x));
+}
+
 int main(int argc, char** argv) {
-  int reps = 200, warmup = 100, gemm_n = 8192, mask = 0;
+  int reps = 200, warmup = 100, gemm_n = 8192, mask = 0, pair = 0;
   size_t elems = (size_t)1 << 28;
   for (int i = 1; i + 1 < argc; i += 2) {
     if (!strcmp(argv[i], "--reps")) reps = atoi(argv[i + 1]);
@@ -101,6 +134,7 @@ int main(int argc, char** argv) {
     else if (!strcmp(argv[i], "--gemm-n")) gemm_n = atoi(argv[i + 1]);
     else if (!strcmp(argv[i], "--triad-elems")) elems = strtoull(argv[i + 1], nullptr, 10);
     else if (!strcmp(argv[i], "--mask")) mask = atoi(argv[i + 1]);
+    else if (!strcmp(argv[i], "--pair")) pair = atoi(argv[i + 1]);
   }
   hipStream_t full = nullptr, masked = nullptr;
   if (orion_stream_create(0, (void**)&full) != ORION_OK) return 3;
@@ -123,11 +157,24 @@ int main(int argc, char** argv) {
   hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)t.c, elems, 4u, 0);
   CHECK(hipStreamSynchronize(full));
 
+  const double flops = 2.0 * gemm_n * (double)gemm_n * gemm_n;
+  if (pair) {
+    float g_ms = 0, t_ms = 0;
+    run_pair(full, masked, &g, &t, 30, 90, &g_ms, &t_ms);  // pilot; settles the clocks
+    run_pair(full, masked, &g, &t, 30, (int)(30 * g_ms / t_ms) + 1, &g_ms, &t_ms);
+    const int n_triad = (int)(reps * g_ms / t_ms) + 1;
+    run_pair(full, masked, &g, &t, reps, n_triad, &g_ms, &t_ms);
+    printf("{\"pair\": true, \"reps\": %d, \"triad_launches\": %d, \"cu_mask\": %d, "
+           "\"gemm\": {\"n\": %d, \"ms\": %.5f, \"tflops\": %.2f, \"frac_of_2500\": %.4f}, "
+           "\"triad\": {\"elems\": %zu, \"ms\": %.5f, \"gbs\": %.1f, \"frac_of_8000\": %.4f}}\n",
+           reps, n_triad, mask, gemm_n, g_ms, flops / g_ms / 1e9, flops / g_ms / 1e9 / 2500.0,
+           elems, t_ms, 12.0 * elems / t_ms / 1e6, 12.0 * elems / t_ms / 1e6 / 8000.0);
+    return 0;
+  }
   const float burst_ms = time_ms(full, 20, 0, launch_gemm, &g);
   const float gemm_ms = time_ms(full, reps, warmup, launch_gemm, &g);
   const float triad_ms = time_ms(masked, reps, 3, launch_triad, &t);
   const float copy_ms = time_ms(full, reps, 3, launch_copy, &t);
-  const double flops = 2.0 * gemm_n * (double)gemm_n * gemm_n;
   printf("{\"reps\": %d, \"warmup\": %d, \"gemm\": {\"n\": %d, \"ms\": %.5f, \"tflops\": %.2f, "
          "\"frac_of_2500\": %.4f, \"burst_ms\": %.5f, \"burst_tflops\": %.2f}, "
          "\"triad\": {\"elems\": %zu, \"cu_mask\": %d, \"ms\": %.5f, \"gbs\": %.1f, \"frac_of_8000\": %.4f}, "
