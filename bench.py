@@ -181,8 +181,11 @@ def main():
         # requests (the high-priority client never idle) and Poisson arrivals
         from orion_amd import kernel_pair as kp_child
         out["kernel_pair_scheduled"] = {}
-        for label, rps in (("closed_loop", 0), ("poisson_400rps", 400)):
-            pair = kp_child.run_child(small=False, check=True, rps=rps,
+        # (the third leg keeps best-effort kernels that alone outlast the budget
+        # off the whole-GPU stream: ORION_CONFINE_LONG_BE=1)
+        for label, rps, confine in (("closed_loop", 0, False), ("poisson_400rps", 400, False),
+                                    ("poisson_400rps_long_be_confined", 400, True)):
+            pair = kp_child.run_child(small=False, check=True, rps=rps, confine_long=confine,
                                       hp_iters=args.pair_requests + 10,
                                       max_be_duration=args.max_be_duration,
                                       workdir=os.path.join(workdir, "pair_" + label))

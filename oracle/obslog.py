@@ -15,7 +15,8 @@ Both logs are line-based text, shared with the native core
 (orion_amd/csrc/policy/obslog.h):
 
 observation log
-    ``J <n> <max_sms> <place_masks comma list>``   job header
+    ``J <n> <max_sms> <place_masks comma list> [L1]``   job header (L1: long
+                                                    best-effort kernels confined)
     ``K <client> <num_kernels> <num_iters> <train 0|1> <profile path>``
     ``X <client> <num_kernels> <profile path>``      setup_change
     ``S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>``
@@ -84,6 +85,7 @@ class RecordingEnv(po.Env):
         self.ops_of = ops_of          # callable(client, op_index) -> OpInfo
         self.algo = algo
         self.budget = None            # Orion's best-effort duration budget (ns)
+        self.confine_long = False     # placement option, header token L1
         self.obs = []
         self.dec = DecisionLog()
         self._reset_poll()
@@ -96,8 +98,10 @@ class RecordingEnv(po.Env):
         self._dec = []
 
     # structure markers -------------------------------------------------
-    def header(self, max_sms, clients):
-        self.obs.append(f"J {self.n} {max_sms} " + ",".join(map(str, self.masks)))
+    def header(self, max_sms, clients, confine_long=False):
+        self.confine_long = bool(confine_long)
+        self.obs.append(f"J {self.n} {max_sms} " + ",".join(map(str, self.masks))
+                        + (" L1" if confine_long else ""))
         for i, (nk, ni, train, path) in enumerate(clients):
             self.obs.append(f"K {i} {nk} {ni} {int(bool(train))} {path}")
 
@@ -161,7 +165,7 @@ class RecordingEnv(po.Env):
             op = self.ops_of(client, op_index)
             cu_slot = place_cu_slot(
                 self.masks, cls, op.sm_used, self.algo, self.hp_active(),
-                self.budget is not None
+                self.confine_long and self.budget is not None
                 and float(op.duration) > float(np.float32(self.budget)))
         self._dec.append(f"D {client} {owner} {cls} {op_index} {event_slot} "
                          f"{cu_slot}")
@@ -242,6 +246,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
     oracle = None
     rec = None
     n = max_sms = masks = None
+    confine_long = False
     clients = {}
     lines = obs_text.splitlines()
     i = 0
@@ -251,6 +256,8 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
         if tag == "J":
             n, max_sms = int(parts[1]), int(parts[2])
             masks = [int(x) for x in parts[3].split(",")]
+            _ensure(len(parts) == 4 or parts[4:] == ["L1"], "J: 3 fields and an optional L1")
+            confine_long = len(parts) == 5
         elif tag == "K":
             clients[int(parts[1])] = (int(parts[2]), int(parts[3]),
                                       bool(int(parts[4])), " ".join(parts[5:]))
@@ -286,6 +293,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
             depth, hp_limit, ustart = int(parts[4]), int(parts[5]), int(parts[6])
             rec.algo = algo
             rec.budget = depth
+            rec.confine_long = confine_long
             rec.dec.add("S")
             oracle.schedule(rec, warmup, witers, algo, depth, hp_limit, ustart,
                             max_polls=len(polls) + 1)

@@ -20,10 +20,11 @@ void appendf(std::string* s, const char* fmt, ...) {
 }
 }  // namespace
 
-void Recorder::header(int max_sms, const std::vector<int>& masks) {
+void Recorder::header(int max_sms, const std::vector<int>& masks, bool confine_long) {
   appendf(&obs_, "J %d %d ", n_, max_sms);
   for (size_t i = 0; i < masks.size(); ++i)
     appendf(&obs_, i ? ",%d" : "%d", masks[i]);
+  if (confine_long) obs_ += " L1";  // long best-effort kernels are confined
   obs_ += '\n';
 }
 
@@ -229,6 +230,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
   };
 
   int n = 0, max_sms = 0;
+  bool confine_long = false;
   std::vector<int> masks;
   std::vector<ClientDesc> clients;
   Policy* policy = nullptr;
@@ -242,8 +244,12 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
     if (l.empty()) continue;
     const char tag = l[0];
     if (tag == 'J') {
-      auto p = split(l, ' ', 4);
-      if (p.size() != 4) { ok = bad(i, "J needs 3 fields"); break; }
+      auto p = split(l, ' ', 5);
+      if (p.size() != 4 && !(p.size() == 5 && p[4] == "L1")) {
+        ok = bad(i, "J needs 3 fields and an optional L1");
+        break;
+      }
+      confine_long = p.size() == 5;
       n = atoi(p[1].c_str());
       max_sms = atoi(p[2].c_str());
       for (auto& m : split(p[3], ',', 1u << 20)) masks.push_back(atoi(m.c_str()));
@@ -290,7 +296,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
         }
         if (!ok) break;
         policy = new Policy(std::move(profs), nk, ni, tr, max_sms, masks,
-                            sequential_fix);
+                            sequential_fix, confine_long);
       }
       ScheduleArgs a;
       a.warmup = atoi(p[1].c_str()) != 0;

@@ -35,7 +35,7 @@ class Recorder : public PolicyHost {
   Recorder(PolicyHost* inner, int n) : inner_(inner), n_(n) {}
   void set_inner(PolicyHost* inner) { inner_ = inner; }
 
-  void header(int max_sms, const std::vector<int>& masks);
+  void header(int max_sms, const std::vector<int>& masks, bool confine_long = false);
   void client(int idx, int num_kernels, int num_iters, bool train,
               const std::string& profile_path);
   void setup_change(int client, int num_kernels, const std::string& path);

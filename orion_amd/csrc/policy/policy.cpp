@@ -134,7 +134,7 @@ static int max_sm_used(const std::vector<OpInfo>& ops) {
 Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
                std::vector<int> num_kernels, std::vector<int> num_iters,
                std::vector<bool> is_train, int max_sms,
-               std::vector<int> cu_masks, bool sequential_fix)
+               std::vector<int> cu_masks, bool sequential_fix, bool confine_long)
     : n_((int)profiles.size()),
       ops_(std::move(profiles)),
       num_kernels_(std::move(num_kernels)),
@@ -143,6 +143,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
       max_sms_(max_sms),
       cu_masks_(std::move(cu_masks)),
       sequential_fix_(sequential_fix),
+      confine_long_(confine_long),
       seen_(n_, 0),
       event_ids_(n_, 0),
       cur_iters_(n_, 0),
@@ -173,7 +174,8 @@ void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class) {
   } else {
     const OpInfo& op = ops_[client][d.op_index];
     d.cu_slot = place_cu_slot(cu_masks_, rec_class, op.sm_used, algo_,
-                              seen_[n_ - 1] > 0, op.duration > (float)be_budget_);
+                              seen_[n_ - 1] > 0,
+                              confine_long_ && op.duration > (float)be_budget_);
   }
   host.dispatch(d);
   if (rec_class == REC_KERNEL) {

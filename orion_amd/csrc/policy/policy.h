@@ -107,7 +107,8 @@ class Policy {
   Policy(std::vector<std::vector<OpInfo>> profiles,
          std::vector<int> num_kernels, std::vector<int> num_iters,
          std::vector<bool> is_train, int max_sms,
-         std::vector<int> cu_masks, bool sequential_fix);
+         std::vector<int> cu_masks, bool sequential_fix,
+         bool confine_long = false);
 
   void setup_change(int client, std::vector<OpInfo> ops, int num_kernels);
 
@@ -138,6 +139,9 @@ class Policy {
   int max_sms_;
   std::vector<int> cu_masks_;
   bool sequential_fix_;
+  // Placement only: a best-effort kernel whose profiled duration alone exceeds
+  // the duration budget is kept off the whole-GPU stream.
+  bool confine_long_;
   // survive between schedule() calls, like the reference's globals
   std::vector<int> seen_;
   std::vector<int> event_ids_;

@@ -425,8 +425,12 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
                           atoi(getenv("ORION_SEQUENTIAL_AS_WRITTEN")) != 0;
   g.n = num_clients;
   g.host.reset();  // streams of a previous job first
+  // Placement option: keep a best-effort kernel that alone outlasts the duration
+  // budget off the whole-GPU stream even while the high-priority client is idle.
+  const bool confine_long = getenv("ORION_CONFINE_LONG_BE") &&
+                            atoi(getenv("ORION_CONFINE_LONG_BE")) != 0;
   g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, cus, g.masks,
-                            !as_written));
+                            !as_written, confine_long));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
   g.host->set_policy(g.policy.get());
   g.recorder.reset();
@@ -435,7 +439,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
     if (*dir) {
       g.record_dir = dir;
       g.recorder.reset(new Recorder(g.host.get(), num_clients));
-      g.recorder->header(cus, g.masks);
+      g.recorder->header(cus, g.masks, confine_long);
       for (int i = 0; i < num_clients; ++i)
         g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
       // start both logs afresh

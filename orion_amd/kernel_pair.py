@@ -199,7 +199,8 @@ def pair_job(small=False, hp_iters=60, rps=0):
 
 
 def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
-              max_be_duration=1_000_000, algo="orion", reef_depth=12, rps=0):
+              max_be_duration=1_000_000, algo="orion", reef_depth=12, rps=0,
+              confine_long=False):
     """Profile both clients and run the pair isolated and co-located, in child
     processes with the interception library preloaded.  Returns the experiment
     summary (see ``colocate.experiment``) plus ``outputs_match`` when ``check``."""
@@ -221,6 +222,8 @@ def run_child(small=False, check=False, workdir=None, hp_iters=60, masks=None,
     extra_env = {}
     if masks:
         extra_env["ORION_BE_CU_MASKS"] = masks
+    if confine_long:
+        extra_env["ORION_CONFINE_LONG_BE"] = "1"
     if check:
         os.makedirs(os.path.join(workdir, "out_iso"), exist_ok=True)
         os.makedirs(os.path.join(workdir, "out_co"), exist_ok=True)

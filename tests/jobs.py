@@ -91,6 +91,7 @@ def make_job(tmp_path, seed, n_clients=2, algo=po.ALGO_ORION, hp_train=False,
     job.traces = traces
     job.arrivals = [rng.randint(20_000, 2_000_000) for _ in range(16)]
     job.closed_loop_hp = rng.random() < 0.3 or hp_train
+    job.confine_long = rng.random() < 0.5
     return job
 
 
@@ -115,7 +116,8 @@ def run_oracle(job, max_polls=3_000_000):
                               hp_active=lambda: oracle.seen[job.n - 1] > 0)
     rec.budget = job.depth
     rec.header(job.max_sms, [(job.nk[c], job.iters[c], job.train[c],
-                              job.paths[c]) for c in range(job.n)])
+                              job.paths[c]) for c in range(job.n)],
+               confine_long=getattr(job, "confine_long", False))
     changes = {1: [(c, po.parse_profile(path), nk, path)
                    for c, (path, nk) in sorted(job.swap.items())]}
     vg.run_job(oracle, env, rec, [(True, 1), (True, 10), (False, 0)],

@@ -68,7 +68,8 @@ def replayed():
     rec = obslog.RecordingEnv(env, 2, masks, lambda c, k: oracle.ops[c][k],
                               algo=po.ALGO_ORION, hp_active=lambda: oracle.seen[1] > 0)
     rec.budget = BUDGET_NS
-    rec.header(256, [(713, 10_000, True, BE), (371, hp_iters, False, HP)])
+    rec.header(256, [(713, 10_000, True, BE), (371, hp_iters, False, HP)],
+               confine_long=True)
     vg.run_job(oracle, env, rec, [(True, 1), (True, 10), (False, 0)], algo=po.ALGO_ORION,
                depth=BUDGET_NS, hp_limit=1, update_start=1, max_polls=30_000_000)
     return oracle, env, rec, hp_iters
@@ -90,8 +91,9 @@ def test_what_the_policy_did_on_that_trace(replayed):
     assert len(hp) == hp_iters * (371 + 2)
     ks = [int(x[4]) for x in hp if x[3] == po.KERNEL]
     assert ks == list(range(371)) * hp_iters
-    # best-effort kernels that alone outlast the budget never got the whole GPU;
-    # short ones did whenever the high-priority client was idle
+    # with the confinement option on (header token L1), best-effort kernels that
+    # alone outlast the budget never got the whole GPU; short ones did whenever
+    # the high-priority client was idle
     be = [x for x in d if x[1] == "0" and x[3] == po.KERNEL]
     long_ops = {k for k, o in enumerate(oracle.ops[0]) if float(o.duration) > BUDGET_NS}
     assert long_ops and all(int(x[6]) < 3 for x in be if int(x[4]) in long_ops)
