@@ -68,6 +68,7 @@ def latency_summary(timings, batch_idx, total_time, train, drop=WARMUP_ITERS):
 
 def write_result(tid, data):
     out_dir = os.environ.get("ORION_RESULT_DIR", ".")
+    os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, f"client_{tid}.json"), "w") as f:
         json.dump(data, f)
 

@@ -114,3 +114,30 @@ def test_order_join_refuses_a_different_kernel_sequence(tmp_path):
     _write_csv(str(tmp_path / "r" / "trace" / "t_kernel_trace.csv"), hdr, rows)
     with pytest.raises(RuntimeError, match="does not end with"):
         rocprof.merge(str(prof), str(tmp_path / "r"), str(tmp_path / "out"))
+
+
+def test_trace_summary_cuts_requests_from_the_end(tmp_path):
+    """Closed form: a thread with 2 + 100 x 3 kernels of 1, 2, 3 us per request
+    (the first two are start-up), another thread with 5 kernels."""
+    from orion_amd.profiling import trace_summary
+    path = tmp_path / "kt_kernel_trace.csv"
+    rows = ["Kind,Agent_Id,Queue_Id,Stream_Id,Thread_Id,Dispatch_Id,Kernel_Id,Kernel_Name,"
+            "Correlation_Id,Start_Timestamp,End_Timestamp"]
+    t = 1000
+    for d in (50_000, 60_000):                      # start-up kernels, cut off
+        rows.append(f"KERNEL_DISPATCH,0,1,0,77,0,0,k,0,{t},{t + d}")
+        t += d + 100
+    for req in range(100):
+        for d in (1000, 2000, 3000):
+            rows.append(f"KERNEL_DISPATCH,0,{1 + req % 2},0,77,0,0,k,0,{t},{t + d}")
+            t += d + 500
+    for i in range(5):
+        rows.append(f"KERNEL_DISPATCH,0,4,0,88,0,0,k,0,{i * 10},{i * 10 + 7}")
+    path.write_text("\n".join(rows) + "\n")
+    s = trace_summary.summarise(str(path), per_request=3, last=40)
+    assert s["77"]["kernels"] == 302 and s["77"]["queues"] == [1, 2]
+    assert s["77"]["groups"] == 40
+    assert s["77"]["kernel_ms"] == {"p50": 0.006, "p99": 0.006, "mean": 0.006}
+    assert s["77"]["span_ms"]["p50"] == 0.007        # 6 us of kernels + two 0.5 us gaps
+    assert abs(s["77"]["sum_ms"] - (0.11 + 100 * 0.006)) < 1e-9
+    assert s["88"] == {"kernels": 5, "sum_ms": 35 / 1e6, "mean_us": 0.007, "queues": [4]}
