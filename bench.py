@@ -41,7 +41,14 @@ WORKLOAD = ("HP: ResNet-50 inference, batch 4, bf16, Poisson arrivals at 80 req/
             "synthetic images N(0,1), labels uniform over 1000 classes, random-init weights")
 
 
-def c3_job(hp_iters):
+def c3_job(hp_iters, hip_graph=False):
+    job = _c3_job(hp_iters)
+    if hip_graph:
+        job[-1]["args"]["hip_graph"] = True
+    return job
+
+
+def _c3_job(hp_iters):
     return [
         {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 1_000_000,
          "args": {"model_name": "resnet50", "batchsize": 32, "rps": 0, "uniform": False,
@@ -52,12 +59,13 @@ def c3_job(hp_iters):
     ]
 
 
-def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False):
+def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_graph=False):
     from orion_amd import colocate
     from orion_amd.profiling import capture_profile
+    os.makedirs(workdir, exist_ok=True)
     cfg = os.path.join(workdir, "job.json")
     with open(cfg, "w") as f:
-        json.dump(c3_job(steps + 10), f)
+        json.dump(c3_job(steps + 10, hip_graph), f)
     job = capture_profile.fill_job(cfg, os.path.join(workdir, "profiles"),
                                    os.path.join(workdir, "job_filled.json"), quiet=True,
                                    use_rocprof=use_rocprof)
@@ -143,6 +151,8 @@ def main():
     ap.add_argument("--kernels-only", action="store_true",
                     help="only the in-process kernel measurements (for profiler runs: "
                          "starts no child process)")
+    ap.add_argument("--no-hip-graph-leg", action="store_true",
+                    help="skip the extra run with a HIP-graph high-priority client")
     ap.add_argument("--pair-requests", type=int, default=300,
                     help="measured GEMM requests of the scheduled kernel pair")
     ap.add_argument("--workdir", default="")
@@ -176,6 +186,20 @@ def main():
         out["config"]["records_per_iteration"] = co["num_kernels"]
         out["colocation_wall_s"] = time.time() - t0
         out["policy_replay"] = policy_replay(os.path.join(workdir, "colocated"))
+        # The same pair with the high-priority client replaying a captured HIP
+        # graph: one copy record and one hipGraphLaunch record per request
+        # instead of 371 kernel records.  (Not the headline: the reference
+        # schedules the request kernel by kernel.)
+        if not args.no_hip_graph_leg:
+            cg = colocation(max(300, args.steps // 2), os.path.join(workdir, "hip_graph"),
+                            args.max_be_duration, args.be_cu_masks, hip_graph=True)
+            out["hp_hip_graph_variant"] = {
+                "isolated_ms": {k: cg["hp_isolated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
+                "colocated_ms": {k: cg["hp_colocated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
+                "p99_ratio": cg["hp_p99_ratio"],
+                "be_colocated_iters_per_s": cg["be_colocated"][0]["throughput"],
+                "be_retained": cg["be_retained"][0],
+                "records_per_iteration": cg["num_kernels"]}
         # configs[1] through the same hot path: GEMM requests (high priority)
         # beside the triad loop (best effort), default CU masks; back-to-back
         # requests (the high-priority client never idle) and Poisson arrivals

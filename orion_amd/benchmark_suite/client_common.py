@@ -25,6 +25,13 @@ WARMUP_ITERS = 10     # iterations before the measured run (:188-198, :220)
 # compared with its isolated run).
 MODEL_INIT_LOCK = threading.RLock()
 
+# One client at a time runs its un-captured set-up (model build, library
+# initialisation, warm-up steps, HIP-graph capture).  A stream capture in one
+# thread makes calls of other threads that touch the legacy stream fail
+# (hipBLASLt's initialisation does: "operation would make the legacy stream
+# depend on a capturing blocking stream"), so the set-up phases must not overlap.
+SETUP_LOCK = threading.RLock()
+
 
 def seed_everything(seed):
     """:22-30."""
@@ -113,9 +120,16 @@ class uncaptured:
         self.backend = backend
 
     def __enter__(self):
+        SETUP_LOCK.acquire()
         self.backend.passthrough(True)
 
     def __exit__(self, *exc):
+        try:
+            self._leave()
+        finally:
+            SETUP_LOCK.release()
+
+    def _leave(self):
         if torch.cuda.is_available():
             torch.cuda.synchronize()
         self.backend.passthrough(False)

@@ -40,12 +40,14 @@ class DummyDataLoader:
 def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                   dummy_data, local_rank, barriers, client_barrier, tid,
                   input_file="", dtype="fp32", momentum=0.9, seed=42,
-                  deterministic=False):
+                  deterministic=False, hip_graph=False):
     cc.seed_everything(seed)
     if deterministic:
         # keep MIOpen off solvers that accumulate with atomics (split-K), whose
         # results differ in the last bit from run to run
         torch.backends.cudnn.deterministic = True
+    if hip_graph and train:
+        raise ValueError("hip_graph is for inference clients")
     backend = cc.Backend()
     sleep_times = cc.arrival_gaps(rps, uniform, num_iters, input_file, seed)
     if not dummy_data:
@@ -87,6 +89,11 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                 loss.backward()
                 optimizer.step()
                 state["loss"] = loss
+            elif "graph" in state:
+                # one copy record and one graph record per request
+                state["graph_in"].copy_(data, non_blocking=True)
+                state["graph"].replay()
+                state["output"] = state["graph_out"]
             else:
                 with torch.no_grad():
                     gpu_data = data.to(device, non_blocking=True).to(tdtype)
@@ -105,6 +112,23 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
         with cc.uncaptured(backend):
             for i in range(cc.UNCAPTURED_STEPS):
                 step(-1 - i)
+            if hip_graph:
+                # The request is launch-bound (hundreds of short kernels): capture
+                # the forward pass once, un-captured by the scheduler, and replay
+                # it per request as a single hipGraphLaunch record.
+                torch.cuda.synchronize()
+                state["graph_in"] = torch.zeros(data.shape, dtype=data.dtype, device=device)
+                graph = torch.cuda.CUDAGraph()
+                # thread_local: what the other clients' threads do meanwhile
+                # (allocations, pinning) is not part of this capture
+                with torch.no_grad(), torch.cuda.graph(graph, stream=stream,
+                                                       capture_error_mode="thread_local"):
+                    state["graph_out"] = model(state["graph_in"].to(tdtype))
+                torch.cuda.synchronize()
+                state["graph"] = graph
+                for i in range(2):
+                    step(-10 - i)
+                torch.cuda.synchronize()
         result = cc.run_client(tid, train, num_iters, sleep_times, barriers, step,
                                backend, extra=extra)
     print(f"Client {tid} finished: {result}", flush=True)

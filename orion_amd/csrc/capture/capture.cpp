@@ -74,6 +74,7 @@ hipStream_t named_stream(const Record& r) {
   if (r.type <= RT_COOP_LAUNCH_KERNEL) return r.u.launch.stream;
   if (r.type <= RT_MODULE_COOP_LAUNCH) return r.u.module.stream;
   if (r.type <= RT_MEMCPY_2D_ASYNC) return r.u.copy.stream;
+  if (r.type == RT_GRAPH_LAUNCH) return r.u.graph.stream;
   if (r.type >= RT_MEMSET) return r.u.set.stream;
   return nullptr;
 }
@@ -191,6 +192,10 @@ int orion_execute_record(const Record* rec, hipStream_t stream) {
       err = hip->hipMemsetD8Async((hipDeviceptr_t)r.u.set.dst,
                                   (unsigned char)r.u.set.value, r.u.set.count,
                                   stream);
+      break;
+    case RT_GRAPH_LAUNCH:
+      err = hip->hipGraphLaunch ? hip->hipGraphLaunch(r.u.graph.exec, stream)
+                                : hipErrorNotSupported;
       break;
     default:
       // reference: "UNSUPPORTED OPERATION - ABORT", utils_sched.cpp:514-516
@@ -470,6 +475,18 @@ hipError_t hipModuleLaunchCooperativeKernel(hipFunction_t f, unsigned int gx,
   Record r;
   r.type = RT_MODULE_COOP_LAUNCH;
   r.u.module = {f, gx, gy, gz, bx, by, bz, shmem, stream, params, nullptr, nullptr, nullptr, 0};
+  return (hipError_t)submit(idx, r, true);
+}
+
+// A captured graph is one record: the policy places and admits it as a whole
+// (its profile row carries the graph's duration), which is what a launch-bound
+// inference client wants -- one hand-off and one launch per request.
+hipError_t hipGraphLaunch(hipGraphExec_t exec, hipStream_t stream) {
+  const int idx = client_for_call(stream);
+  if (idx < 0) return orion_hip_api()->hipGraphLaunch(exec, stream);
+  Record r;
+  r.type = RT_GRAPH_LAUNCH;
+  r.u.graph = {exec, stream};
   return (hipError_t)submit(idx, r, true);
 }
 

@@ -45,13 +45,14 @@ enum RecType : int32_t {
   RT_MEMSET_D32_ASYNC,         // hipMemsetD32Async
   RT_MEMSET_D16_ASYNC,         // hipMemsetD16Async
   RT_MEMSET_D8_ASYNC,          // hipMemsetD8Async
+  RT_GRAPH_LAUNCH,             // hipGraphLaunch: a whole captured graph, one record
   RT_COUNT
 };
 
 // Policy class of a record type (reference: which cases of schedule_kernel bump
 // `seen`, src/scheduler/utils_sched.cpp:242-513).
 inline int rec_class_of(int type) {
-  if (type <= RT_MODULE_COOP_LAUNCH) return REC_KERNEL;
+  if (type <= RT_MODULE_COOP_LAUNCH || type == RT_GRAPH_LAUNCH) return REC_KERNEL;
   if (type <= RT_MEMCPY_2D_ASYNC) return REC_MEMCPY;
   if (type == RT_MALLOC) return REC_MALLOC;
   if (type == RT_FREE) return REC_FREE;
@@ -113,6 +114,10 @@ struct Record {
       size_t count;  // bytes, or elements for the D32/D16/D8 forms
       hipStream_t stream;
     } set;
+    struct {
+      hipGraphExec_t exec;
+      hipStream_t stream;
+    } graph;
   } u;
 };
 

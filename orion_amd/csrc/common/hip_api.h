@@ -68,6 +68,7 @@ namespace orion {
   X(hipMemsetD32Async, hipError_t, (hipDeviceptr_t, int, size_t, hipStream_t))              \
   X(hipMemsetD16Async, hipError_t, (hipDeviceptr_t, unsigned short, size_t, hipStream_t))   \
   X(hipMemsetD8Async, hipError_t, (hipDeviceptr_t, unsigned char, size_t, hipStream_t))     \
+  X(hipGraphLaunch, hipError_t, (hipGraphExec_t, hipStream_t))                              \
   X(hipStreamSynchronize, hipError_t, (hipStream_t))                                        \
   X(hipStreamQuery, hipError_t, (hipStream_t))                                              \
   X(hipStreamWaitEvent, hipError_t, (hipStream_t, hipEvent_t, unsigned int))                \

@@ -87,6 +87,14 @@ void describe(const Record& r, Row* row, const HipApi* hip, hipStream_t stream) 
   row->type = r.type;
   row->regs = 0;
   row->static_lds = 0;
+  if (r.type == RT_GRAPH_LAUNCH) {
+    // a whole captured graph: no single grid; the profile writer gives it
+    // every compute unit and an unknown class
+    row->gx = row->gy = row->gz = row->bx = row->by = row->bz = 0;
+    row->shmem = 0;
+    row->name = "hipGraphLaunch";
+    return;
+  }
   if (r.type <= RT_COOP_LAUNCH_KERNEL) {
     row->gx = r.u.launch.grid.x; row->gy = r.u.launch.grid.y; row->gz = r.u.launch.grid.z;
     row->bx = r.u.launch.block.x; row->by = r.u.launch.block.y; row->bz = r.u.launch.block.z;

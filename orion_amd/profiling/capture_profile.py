@@ -28,6 +28,7 @@ from .. import scheduler_frontend as fe
 from . import cu_need
 
 HEADER = "Name,Profile,Memory_footprint,SM_usage,Duration"
+GRAPH_LAUNCH = "hipGraphLaunch"      # name the capture gives a hipGraphLaunch record
 
 
 def read_trace(path):
@@ -45,6 +46,11 @@ def profile_rows(reference_iter, all_iters):
     same = [it for it in all_iters if [r["name"] for r in it] == names]
     out = []
     for i, r in enumerate(reference_iter):
+        if r["name"] == GRAPH_LAUNCH:
+            # a whole captured graph is one record: every CU, class unknown
+            dur = statistics.median(float(it[i]["duration_ns"]) for it in same)
+            out.append((r["name"], -1, 0, cu_need.TOTAL_CUS, max(1, int(round(dur)))))
+            continue
         threads = int(r["block_x"]) * int(r["block_y"]) * int(r["block_z"])
         blocks = int(r["grid_x"]) * int(r["grid_y"]) * int(r["grid_z"])
         lds = int(r["dyn_lds"]) + int(r["static_lds"])

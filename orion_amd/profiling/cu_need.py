@@ -21,6 +21,7 @@ VGPRS_PER_SIMD = 512
 VGPR_GRANULE = 8
 LDS_PER_CU = 160 * 1024
 MAX_WORKGROUPS_PER_CU = 32
+TOTAL_CUS = 256                # MI355X
 
 
 def workgroups_per_cu(threads_per_block, regs_per_thread=0, lds_per_block=0):

@@ -2,7 +2,10 @@
 against the recording HIP stand-in (tests/fakehip).  Runs in its own process
 (the HIP table of a process is resolved once); prints one JSON object.
 
-usage: python tests/fake_runner.py <workdir> <algo> <n_be> <hp_iters>
+usage: python tests/fake_runner.py <workdir> <algo> <n_be> <hp_iters> [graph]
+
+With ``graph`` the high-priority client submits each iteration's kernels as one
+executable graph (hipGraphLaunch): one kernel-class record per iteration.
 """
 
 import ctypes
@@ -20,6 +23,7 @@ import numpy as np  # noqa: E402
 from orion_amd import _lib, scheduler_frontend as fe  # noqa: E402
 
 workdir, algo, n_be, hp_iters = sys.argv[1], sys.argv[2], int(sys.argv[3]), int(sys.argv[4])
+hp_graph = len(sys.argv) > 5 and sys.argv[5] == "graph"
 os.environ["ORION_RECORD_DIR"] = workdir
 os.environ["ORION_QUIET"] = "1"
 
@@ -38,9 +42,20 @@ cap.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
 cap.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
 cap.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 
+cap.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+
+
+class FakeGraphExec(ctypes.Structure):      # mirrors tests/fakehip/fakehip.cpp
+    _fields_ = [("n", ctypes.c_int), ("fn", ctypes.c_void_p * 8),
+                ("params", ctypes.POINTER(ctypes.c_void_p) * 8)]
+
+
 N = 64
 n_clients = n_be + 1
-kernels_per_iter = [5 + c for c in range(n_clients)]
+kernels_per_iter = [5 + c for c in range(n_clients)]      # what an iteration computes
+records_per_iter = list(kernels_per_iter)                 # what the scheduler counts
+if hp_graph:
+    records_per_iter[-1] = 1
 iters = [10_000] * n_be + [hp_iters]
 
 
@@ -56,7 +71,7 @@ def write_profile(path, nk, seed):
 files = []
 for c in range(n_clients):
     p = os.path.join(workdir, f"client{c}.csv")
-    write_profile(p, kernels_per_iter[c], c)
+    write_profile(p, records_per_iter[c], c)
     files.append(p)
 
 results = [None] * n_clients
@@ -64,10 +79,13 @@ iters_done = [0] * n_clients
 barriers = [threading.Barrier(n_clients + 1)]
 
 
+def param_array(params):
+    return (ctypes.c_void_p * len(params))(*[ctypes.cast(ctypes.pointer(p), ctypes.c_void_p)
+                                             for p in params])
+
+
 def launch(func, params):
-    arr = (ctypes.c_void_p * len(params))(*[ctypes.cast(ctypes.pointer(p), ctypes.c_void_p)
-                                            for p in params])
-    rc = cap.hipModuleLaunchKernel(func, 1, 1, 1, 64, 1, 1, 0, None, arr, None)
+    rc = cap.hipModuleLaunchKernel(func, 1, 1, 1, 64, 1, 1, 0, None, param_array(params), None)
     assert rc == 0, rc
 
 
@@ -83,9 +101,20 @@ def client(tid):
     it = 0
     n_c, a_c = ctypes.c_int(N), ctypes.c_float(0.5)
     c_c = ctypes.c_float(0.125)
+    graph = None
+    if hp_graph and tid == n_clients - 1:
+        graph, keep = FakeGraphExec(), []
+        graph.n = nk
+        for k in range(nk):
+            arr = param_array([dev_y, dev_x, a_c, n_c] if k % 2 == 0 else [dev_y, c_c, n_c])
+            keep.append(arr)
+            graph.fn[k] = SAXPY if k % 2 == 0 else SQADD
+            graph.params[k] = ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p))
     while it < iters[tid]:
         cap.hipMemcpyAsync(dev_x, host_x.ctypes.data, N * 4, 1, None)
-        for k in range(nk):
+        if graph is not None:
+            assert cap.hipGraphLaunch(ctypes.byref(graph), None) == 0
+        for k in range(nk if graph is None else 0):
             if k % 2 == 0:
                 launch(SAXPY, [dev_y, dev_x, a_c, n_c])
             else:
@@ -128,7 +157,7 @@ sched_tid = []
 def run_sched():
     sched_tid.append(threading.get_native_id())
     py.run_scheduler(barriers, tids, ["fake"] * n_clients, files,
-                     [None] * n_clients, kernels_per_iter, [None] * n_clients,
+                     [None] * n_clients, records_per_iter, [None] * n_clients,
                      iters, True, True, algo == "reef", algo == "sequential",
                      8 if algo == "reef" else 100_000, 1, 1, [True] * n_be + [False])
 

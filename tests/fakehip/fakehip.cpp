@@ -170,6 +170,20 @@ hipError_t hipModuleLaunchCooperativeKernel(hipFunction_t f, unsigned int gx,
                                             hipStream_t s, void** params) {
   return hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, shmem, s, params, nullptr);
 }
+// A stand-in executable graph: up to eight host kernels run in order, logged as
+// one launch (kind 0) like any other kernel.
+struct FakeGraphExec {
+  int n;
+  fake_kernel_t fn[8];
+  void** params[8];
+};
+hipError_t hipGraphLaunch(hipGraphExec_t exec, hipStream_t s) {
+  FakeGraphExec* g = (FakeGraphExec*)exec;
+  log_call(0, s, (uint64_t)exec, (uint64_t)g->n);
+  for (int i = 0; i < g->n; ++i) g->fn[i](g->params[i]);
+  occupy(s, g_kernel_ns * g->n);
+  return hipSuccess;
+}
 hipError_t hipMalloc(void** p, size_t n) {
   *p = malloc(n ? n : 1);
   log_call(3, nullptr, (uint64_t)*p, n);

@@ -33,12 +33,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FAKEHIP = os.path.join(ROOT, "tests", "fakehip", "libfakehip.so")
 
 
-def run_child(workdir, algo, n_be, hp_iters, direct=True):
+def run_child(workdir, algo, n_be, hp_iters, direct=True, graph=False):
     if not os.path.exists(FAKEHIP):
         pytest.fail("tests/fakehip/libfakehip.so is not built (make -C orion_amd/csrc)")
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), workdir,
-         algo, str(n_be), str(hp_iters)],
+         algo, str(n_be), str(hp_iters)] + (["graph"] if graph else []),
         capture_output=True, text=True, timeout=300,
         env=dict(os.environ, ORION_HP_DIRECT="1" if direct else "0"))
     assert proc.returncode == 0, proc.stdout + proc.stderr
@@ -78,3 +78,24 @@ def test_job_protocol_on_fake_runtime(tmp_path, algo, n_be, direct):
     assert dec.count("\nD ") > 100
     assert obslog.replay(obs) == dec            # CPU oracle, bit-exact
     assert jobs.native_replay(obs) == dec       # native core, replayed
+
+
+@pytest.mark.parametrize("direct", [True, False])
+def test_a_captured_graph_is_one_record(tmp_path, direct):
+    """The high-priority client submits every iteration as one executable graph
+    (hipGraphLaunch): the scheduler counts one kernel-class record per iteration,
+    the result is the same, the log replays bit-exactly."""
+    hp_iters = 30
+    res = run_child(str(tmp_path), "orion", 2, hp_iters, direct, graph=True)
+    assert not any(res["alive"])
+    assert res["iters_done"][-1] == hp_iters and all(res["outputs_equal"]), res
+    hp_tid, sched = res["client_tids"][-1], res["sched_tid"][0]
+    issuer = str(hp_tid if direct else sched)
+    assert issuer in res["launches_by_tid"]
+    if direct:      # one launch per iteration, all but the first by the client itself
+        assert hp_iters - 1 <= res["launches_by_tid"][str(hp_tid)] <= hp_iters
+    obs = open(os.path.join(str(tmp_path), "observations.log")).read()
+    dec = open(os.path.join(str(tmp_path), "decisions.log")).read()
+    hp = [l.split() for l in dec.splitlines() if l.startswith(f"D 2 ")]
+    assert sum(1 for x in hp if x[3] == "k") == hp_iters      # one kernel record each
+    assert obslog.replay(obs) == dec and jobs.native_replay(obs) == dec

@@ -215,3 +215,73 @@ def test_four_clients_round_robin(tmp_path):
                          torch.tensor(float(torch.tensor(1.7, dtype=torch.float32)),
                                       dtype=torch.float64, device="cuda:0")).float().cpu()
     assert torch.equal(out, want)
+
+
+def test_hip_graph_replays_match_eager_every_time():
+    """The HIP-graph request path (train_imagenet.py, hip_graph) replays one
+    captured forward pass per request.  Replays of a captured graph must be
+    checked one by one, with ordinary work and synchronisations between them:
+    every replay against the eager result for the same input, and against the
+    CPU fp32 reference."""
+    from orion_amd.benchmark_suite import client_common as cc
+    from orion_amd.benchmark_suite.vision_models import resnet50
+    with cc.MODEL_INIT_LOCK:
+        cc.seed_everything(42)
+        cpu_model = resnet50().eval()
+    model = copy.deepcopy(cpu_model).cuda()
+    stream = torch.cuda.Stream()
+    gen = torch.Generator().manual_seed(7)
+    with torch.cuda.stream(stream), torch.no_grad():
+        static_in = torch.zeros(4, 3, 224, 224, device="cuda")
+        for _ in range(3):
+            model(static_in)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream, capture_error_mode="thread_local"):
+            static_out = model(static_in)
+        torch.cuda.synchronize()
+        for i in range(6):
+            x = torch.randn(4, 3, 224, 224, generator=gen)
+            eager = model(x.cuda()).float().cpu()
+            static_in.copy_(x, non_blocking=True)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = static_out.float().cpu()
+            ref = cpu_model(x)
+            scale = ref.abs().max()
+            assert float((got - ref).abs().max() / scale) <= CPU_RTOL, i
+            assert float((got - eager).abs().max() / scale) <= CPU_RTOL, i
+            _ = (x.cuda() * 2).sum().item()          # eager work between replays
+
+
+def test_hip_graph_client_beside_a_trainer(tmp_path):
+    """A launch-bound inference client that replays a captured HIP graph: one
+    copy record and one hipGraphLaunch record per request through the same hot
+    path, beside a best-effort trainer."""
+    job = [
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": True}},
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 60,
+         "args": {"model_name": "resnet50", "batchsize": 4, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": False, "dtype": "fp32", "hip_graph": True}},
+    ]
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job)
+    assert filled[-1]["num_kernels"] == 1           # the graph is one record
+    assert open(filled[-1]["kernel_file"]).read().splitlines()[1].startswith("hipGraphLaunch,-1,0,256,")
+    assert co[-1]["iterations"] == 60 and co[0]["iterations"] >= 10
+    from orion_amd.benchmark_suite import client_common as cc
+    from orion_amd.benchmark_suite.train_imagenet import DummyDataLoader
+    from orion_amd.benchmark_suite.vision_models import resnet50
+    with cc.MODEL_INIT_LOCK:
+        cc.seed_everything(42)
+        model = resnet50().eval()
+    data, _ = next(DummyDataLoader(4, 42))
+    with torch.no_grad():
+        ref = model(data.float())
+    scale = ref.abs().max()
+    assert float((co_out - ref).abs().max() / scale) <= CPU_RTOL
+    assert float((iso_out - co_out).abs().max() / scale) <= CPU_RTOL
+    dec = _check_replay(co_dir)
+    hp_kernels = [l for l in dec.splitlines() if l.startswith("D 1 1 k")]
+    assert len(hp_kernels) == 60
