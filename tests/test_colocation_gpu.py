@@ -117,7 +117,7 @@ def test_resnet50_colocation_outputs_and_replay(tmp_path):
     _check_replay(co_dir)
 
 
-def _run_iso_and_co(work, job, budget=160000):
+def _run_iso_and_co(work, job, budget=160000, extra_env=None):
     """Profiles the job's clients, runs the high-priority client alone and the
     whole job, both saving outputs; returns (filled job, co-located results,
     isolated HP output, co-located HP output, record dir)."""
@@ -131,11 +131,12 @@ def _run_iso_and_co(work, job, budget=160000):
     iso_dir, co_dir = os.path.join(work, "iso_out"), os.path.join(work, "co_out")
     os.makedirs(iso_dir)
     os.makedirs(co_dir)
+    extra_env = dict(extra_env or {})
     colocate.run_job([copy.deepcopy(filled[-1])], "orion", os.path.join(work, "iso"),
-                     budget, env={"ORION_SAVE_OUTPUT_DIR": iso_dir})
+                     budget, env=dict(extra_env, ORION_SAVE_OUTPUT_DIR=iso_dir))
     co = colocate.run_job(copy.deepcopy(filled), "orion", os.path.join(work, "co"),
-                          budget, env={"ORION_SAVE_OUTPUT_DIR": co_dir,
-                                       "ORION_RECORD_DIR": co_dir})
+                          budget, env=dict(extra_env, ORION_SAVE_OUTPUT_DIR=co_dir,
+                                           ORION_RECORD_DIR=co_dir))
     hp = len(job) - 1
     iso_out = torch.load(os.path.join(iso_dir, "client_0_output.pt"), weights_only=True)
     co_out = torch.load(os.path.join(co_dir, f"client_{hp}_output.pt"), weights_only=True)
@@ -254,10 +255,12 @@ def test_hip_graph_replays_match_eager_every_time():
             _ = (x.cuda() * 2).sum().item()          # eager work between replays
 
 
-def test_hip_graph_client_beside_a_trainer(tmp_path):
+@pytest.mark.parametrize("direct", ["1", "0"])
+def test_hip_graph_client_beside_a_trainer(tmp_path, direct):
     """A launch-bound inference client that replays a captured HIP graph: one
     copy record and one hipGraphLaunch record per request through the same hot
-    path, beside a best-effort trainer."""
+    path, beside a best-effort trainer -- issued by the client itself (default)
+    or handed to the scheduler thread (ORION_HP_DIRECT=0)."""
     job = [
         {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
          "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
@@ -266,7 +269,8 @@ def test_hip_graph_client_beside_a_trainer(tmp_path):
          "args": {"model_name": "resnet50", "batchsize": 4, "rps": 0, "uniform": False,
                   "dummy_data": True, "train": False, "dtype": "fp32", "hip_graph": True}},
     ]
-    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job)
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(
+        str(tmp_path), job, extra_env={"ORION_HP_DIRECT": direct})
     assert filled[-1]["num_kernels"] == 1           # the graph is one record
     assert open(filled[-1]["kernel_file"]).read().splitlines()[1].startswith("hipGraphLaunch,-1,0,256,")
     assert co[-1]["iterations"] == 60 and co[0]["iterations"] >= 10
