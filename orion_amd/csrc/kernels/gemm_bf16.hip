@@ -49,13 +49,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
-
 // c += a * b on the matrix core; c lives in accumulator registers and is
 // updated in place (as a builtin call the register allocator shuffles the 256
 // accumulators between register files in every iteration).
@@ -63,9 +56,21 @@ __device__ __forceinline__ void mfma_16x16x32(f32x4& c, const bf16x8& a, const b
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
-__device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
-__device__ __forceinline__ void store_out(uint16_t* p, float v) {
-  *p = f32_to_bf16_rne(v);
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Four consecutive elements of a row of C from one accumulator tile.
+__device__ __forceinline__ void store_quad(float* p, const f32x4& v) {
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+// bf16: round to nearest even (v_cvt_pk_bf16_f32 on gfx950), two per register.
+__device__ __forceinline__ void store_quad(uint16_t* p, const f32x4& v) {
+  const f32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+  u32x2 packed;
+  packed[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+  packed[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+  *reinterpret_cast<u32x2*>(p) = packed;
 }
 
 // Workgroup id -> output tile.  Hardware hands consecutive workgroup ids to the
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_bf16_nt_kernel(
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < 64; ++m) {
-      mfma_16x16x32(acc[m >> 3][m & 7], fa[0][m >> 3], fb[0][m & 7]);
+      mfma_16x16x32(acc[m >> 3][m & 7], fb[0][m & 7], fa[0][m >> 3]);
       read_slot(KS1{}, cur, m);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_bf16_nt_kernel(
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < 64; ++m) {
-      mfma_16x16x32(acc[m >> 3][m & 7], fa[1][m >> 3], fb[1][m & 7]);
+      mfma_16x16x32(acc[m >> 3][m & 7], fb[1][m & 7], fa[1][m >> 3]);
       if (kNext) read_slot(KS0{}, nxt, m);
       if (kLoads && (m & 3) == 2) load_one(kt + 2, cur, m >> 2);
       __builtin_amdgcn_sched_barrier(0);
@@ -234,46 +239,45 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_bf16_nt_kernel(
   // ones time to write their accumulators before anything reads them.
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-  // Epilogue.  Accumulator register r of a 16x16 tile holds row lq*4 + r,
-  // column l16: stored as it lies, a lane would write two bytes at a time in
-  // 32-byte runs.  Each wave instead turns its 128 x 128 block round in its own
-  // quarter of the LDS (free now) and writes whole rows, 16 bytes per lane, so
-  // every store instruction covers full cache lines.  A row is cut into eight
-  // chunks of 16 elements; chunk j of row R sits at position j ^ ((R >> 2) & 3),
-  // which spreads the four row groups of one write over all banks.
+  // Epilogue.  The MFMAs ran with the B fragment as first operand, so a lane's
+  // four accumulators of tile (i, j) are four CONSECUTIVE columns of one row of
+  // C: row i*16 + l16, columns j*16 + lq*4 .. +3.  They are converted, packed
+  // and written as one 8- or 16-byte piece into the wave's own quarter of the
+  // LDS (free now); whole rows are then read back and stored 16 bytes per lane,
+  // so every store instruction covers full cache lines.  A row is cut into
+  // 16-byte slots; slot s of row R sits at s ^ (R & 15), which keeps the sixteen
+  // rows one write instruction touches apart.
   __builtin_amdgcn_s_waitcnt(0xc07f);
   __builtin_amdgcn_s_barrier();  // every wave has read its last fragments
   constexpr int kElt = (int)sizeof(OutT);
   constexpr int kRowB = 128 * kElt;          // bytes of one row of the block
-  constexpr int kChunkB = 16 * kElt;
   constexpr int kPassRows = 32768 / kRowB;   // rows that fit the wave's quarter
   constexpr int kPasses = 128 / kPassRows;   // 1 (bf16) or 2 (fp32)
   constexpr int kIPerPass = 8 / kPasses;
-  constexpr int kUnits = kRowB / 16;         // 16-byte units per row
-  constexpr int kRowsPerStore = 64 / kUnits;
+  constexpr int kSlots = kRowB / 16;         // 16-byte slots per row
+  constexpr int kRowsPerStore = 64 / kSlots;
   unsigned char* ep = lds + wave * 32768;
-  const int st_row = lane / kUnits;
-  const int st_unit = lane % kUnits;
+  const int st_row = lane / kSlots;
+  const int st_slot = lane % kSlots;
   OutT* c_block = C + (row0_a + wm * 128) * (size_t)N + row0_b + wn * 128;
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
     for (int ii = 0; ii < kIPerPass; ++ii)
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          store_out(reinterpret_cast<OutT*>(ep + (ii * 16 + lq * 4 + r) * kRowB +
-                                            (j ^ lq) * kChunkB) + l16,
-                    acc[pass * kIPerPass + ii][j][r]);
+      for (int j = 0; j < 8; ++j) {
+        const int byte = (j * 16 + lq * 4) * kElt;
+        unsigned char* dst = ep + (ii * 16 + l16) * kRowB +
+                             (((byte >> 4) ^ l16) << 4) + (byte & 15);
+        store_quad(reinterpret_cast<OutT*>(dst), acc[pass * kIPerPass + ii][j]);
+      }
 #pragma unroll
     for (int it = 0; it < kPassRows / kRowsPerStore; ++it) {
       const int R = it * kRowsPerStore + st_row;
-      const int byte = st_unit * 16;
-      const int phys = ((byte / kChunkB) ^ ((R >> 2) & 3)) * kChunkB + byte % kChunkB;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(ep + R * kRowB + phys);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(ep + R * kRowB +
+                                                      ((st_slot ^ (R & 15)) << 4));
       __builtin_nontemporal_store(
-          v, reinterpret_cast<u32x4*>(c_block + (size_t)(pass * kPassRows + R) * N) + st_unit);
+          v, reinterpret_cast<u32x4*>(c_block + (size_t)(pass * kPassRows + R) * N) + st_slot);
     }
   }
 }
