@@ -32,7 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 # profiles/bench_kernels_gemm8192_triad1GiB_counters.txt
-GEMM_TRAFFIC_BYTES = int((786999.1 * 2.0 + 131084.6 * 1.0) * 1024)
+GEMM_TRAFFIC_BYTES = int((786877.9 * 2.0 + 131106.5 * 1.0) * 1024)
 TRIAD_TRAFFIC_BYTES = int((1048588.2 * 2.0 + 1048576.1 * 1.0) * 1024)
 
 METRIC = "HP p99 latency vs isolated + BE iters/sec retained, co-located on 1 MI355X"
