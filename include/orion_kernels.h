@@ -28,8 +28,8 @@ enum orion_status {
 /* a[i] = fmaf(s, c[i], b[i]) for i in [0, n): one fused multiply-add per
  * element, so results are bit-identical to C's fmaf on the host.
  * grid_blocks <= 0 selects the default launch (one 16-byte access per lane,
- * n / 1024 workgroups of 256 lanes); a smaller positive value is honoured with
- * block-contiguous chunks.  ORION_ERR_SHAPE if n needs more than 2^31 - 1
+ * n / 256 workgroups of one 64-lane wavefront); a smaller positive value is
+ * honoured with block-contiguous chunks of 256-lane workgroups.  ORION_ERR_SHAPE if n needs more than 2^31 - 1
  * workgroups.
  * Memory-bound stand-in for bnorm_trainer.py:20-27 of the reference. */
 int orion_triad_f32(float* a, const float* b, const float* c, float s,

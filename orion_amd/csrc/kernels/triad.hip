@@ -5,10 +5,11 @@
 // (global_load_dwordx4 / global_store_dwordx4, non-temporal: nothing is reused),
 // so a wavefront touches one fully coalesced 1 KiB segment per access.
 //
-// Default launch: one 16-byte access per lane and array, i.e. n / 1024
-// workgroups with no loop.  On MI355X this shape streams fastest -- the
-// dispatcher keeps every CU's memory pipeline full with short-lived waves
-// (measured over 3 x 1 GiB: 6.4 TB/s against 4.6 TB/s for a 2048-workgroup
+// Default launch: one 16-byte access per lane and array and one wavefront per
+// workgroup, i.e. n / 256 workgroups with no loop.  On MI355X this shape streams
+// fastest -- the dispatcher keeps every CU's memory pipeline full with
+// short-lived waves (measured over 3 x 1 GiB: 6.72 TB/s; 6.43 TB/s with four
+// waves per workgroup, 6.4 with two accesses per lane, 4.6 for a 2048-workgroup
 // grid-stride loop with four accesses in flight per lane).  A caller-chosen
 // smaller grid walks block-contiguous chunks instead, so any number of compute
 // units (a CU-masked stream may expose a fraction of the 256) drains it.
@@ -24,7 +25,8 @@
 
 namespace {
 
-constexpr int kTriadThreads = 256;
+constexpr int kTriadThreads = 256;  // chunked variant
+constexpr int kOneShotThreads = 64; // one-shot variant: one wavefront per workgroup
 // float4 accesses in flight per lane and per array in the chunked variant.
 constexpr int kTriadUnroll = 4;
 
@@ -49,10 +51,10 @@ __device__ __forceinline__ void triad_tail(float* a, const float* b, const float
   }
 }
 
-__global__ __launch_bounds__(kTriadThreads) void triad_f32_kernel(
+__global__ __launch_bounds__(kOneShotThreads) void triad_f32_kernel(
     float* __restrict__ a, const float* __restrict__ b,
     const float* __restrict__ c, float s, size_t n_vec4, size_t n) {
-  const size_t i = (size_t)blockIdx.x * kTriadThreads + threadIdx.x;
+  const size_t i = (size_t)blockIdx.x * kOneShotThreads + threadIdx.x;
   if (i < n_vec4) {
     const f32x4 vb = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(b) + i);
     const f32x4 vc = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(c) + i);
@@ -100,11 +102,11 @@ extern "C" int orion_triad_f32(float* a, const float* b, const float* c,
   if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) != 0)
     return ORION_ERR_ALIGN;
   const size_t n_vec4 = n / 4;
-  size_t one_shot = (n_vec4 + kTriadThreads - 1) / kTriadThreads;
+  size_t one_shot = (n_vec4 + kOneShotThreads - 1) / kOneShotThreads;
   if (one_shot < 1) one_shot = 1;
   if (one_shot > 0x7fffffffu) return ORION_ERR_SHAPE;
   if (grid_blocks <= 0 || (size_t)grid_blocks >= one_shot) {
-    hipLaunchKernelGGL(triad_f32_kernel, dim3((unsigned)one_shot), dim3(kTriadThreads), 0,
+    hipLaunchKernelGGL(triad_f32_kernel, dim3((unsigned)one_shot), dim3(kOneShotThreads), 0,
                        (hipStream_t)stream, a, b, c, s, n_vec4, n);
   } else {
     hipLaunchKernelGGL(triad_f32_chunked_kernel, dim3((unsigned)grid_blocks),
