@@ -56,6 +56,9 @@ kernels_per_iter = [5 + c for c in range(n_clients)]      # what an iteration co
 records_per_iter = list(kernels_per_iter)                 # what the scheduler counts
 if hp_graph:
     records_per_iter[-1] = 1
+if os.environ.get("FAKE_RUNNER_MISCOUNT"):
+    # tell the scheduler one kernel more than client 0 submits per iteration
+    records_per_iter[0] += 1
 iters = [10_000] * n_be + [hp_iters]
 
 

@@ -99,3 +99,20 @@ def test_a_captured_graph_is_one_record(tmp_path, direct):
     hp = [l.split() for l in dec.splitlines() if l.startswith(f"D 2 ")]
     assert sum(1 for x in hp if x[3] == "k") == hp_iters      # one kernel record each
     assert obslog.replay(obs) == dec and jobs.native_replay(obs) == dec
+
+
+def test_kernel_count_mismatch_ends_the_job_with_a_report(tmp_path):
+    """The reference spins forever when a client submits fewer kernels per
+    iteration than its profile names (scheduler_eval.cpp:282, :389).  Here the
+    scheduler notices that nothing is dispatched or completed while a client
+    waits, prints what it sees per client and aborts."""
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), str(tmp_path),
+         "orion", "1", "20"],
+        capture_output=True, text=True, timeout=120,
+        env=dict(os.environ, FAKE_RUNNER_MISCOUNT="1", ORION_STUCK_LIMIT_S="1"))
+    assert proc.returncode != 0
+    assert "kernel count probably differs" in proc.stderr
+    # client 0 has handed over all 5 of the 6 kernels the scheduler was told about
+    assert "client 0: 5 of 6 kernel records seen this iteration" in proc.stderr
+    assert "block() calls 1, iterations released 0" in proc.stderr
