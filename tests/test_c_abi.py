@@ -58,6 +58,7 @@ def test_interposed_hip_symbols_are_exported():
     for n in ("hipLaunchKernel", "hipExtLaunchKernel", "hipModuleLaunchKernel",
               "hipExtModuleLaunchKernel", "hipHccModuleLaunchKernel",
               "hipModuleLaunchCooperativeKernel", "hipLaunchCooperativeKernel",
+              "hipGraphLaunch",
               "hipMalloc", "hipFree", "hipMemcpy", "hipMemcpyAsync",
               "hipMemcpyWithStream", "hipMemcpy2DAsync", "hipMemset",
               "hipMemsetAsync", "hipMemsetD32Async", "hipMemsetD16Async",
