@@ -30,8 +30,11 @@ def preload_env(extra=None):
 
 
 def run_job(job, algo, workdir, max_be_duration, reef_depth=12, env=None,
-            timeout=900, log_name="launch.log"):
-    """One launcher process; returns the list of client result dicts."""
+            timeout=900, log_name="launch.log", hp_limit=None, start_update=None):
+    """One launcher process; returns the list of client result dicts.
+    ``hp_limit`` (ms) and ``start_update`` (kernel index) are the launcher's
+    --orion_hp_limit / --orion_start_update, used when the high-priority client
+    trains."""
     os.makedirs(workdir, exist_ok=True)
     cfg = os.path.join(workdir, "job.json")
     with open(cfg, "w") as f:
@@ -41,6 +44,10 @@ def run_job(job, algo, workdir, max_be_duration, reef_depth=12, env=None,
     cmd = [sys.executable, "-u", "-m", "orion_amd.launch_jobs", "--algo", algo,
            "--config_file", cfg, "--orion_max_be_duration", str(max_be_duration),
            "--reef_depth", str(reef_depth)]
+    if hp_limit is not None:
+        cmd += ["--orion_hp_limit", str(hp_limit)]
+    if start_update is not None:
+        cmd += ["--orion_start_update", str(start_update)]
     with open(os.path.join(workdir, log_name), "w") as log:
         proc = subprocess.run(cmd, stdout=log, stderr=subprocess.STDOUT, env=e,
                               timeout=timeout,

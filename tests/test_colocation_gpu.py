@@ -292,3 +292,37 @@ def test_hip_graph_client_beside_a_trainer(tmp_path, direct):
     dec = _check_replay(co_dir)
     hp_kernels = [l for l in dec.splitlines() if l.startswith("D 1 1 k")]
     assert len(hp_kernels) == 60
+
+
+def test_high_priority_training_client(tmp_path):
+    """The high-priority client trains (reference: scheduler_eval.cpp:266-275,
+    :338, :427-445): best-effort work is held to half the CU need of the
+    best-effort profile, re-tuned from the measured iteration time against
+    --orion_hp_limit, and admitted freely once the optimizer update has begun
+    (--orion_start_update).  Such a client always hands its records over."""
+    from orion_amd import colocate
+    from orion_amd.profiling import capture_profile
+    work = str(tmp_path)
+    job = [
+        {"arch": "mobilenet_v2", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"model_name": "mobilenet_v2", "batchsize": 16, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": True}},
+        {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 45,
+         "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": True}},
+    ]
+    cfg = os.path.join(work, "job.json")
+    with open(cfg, "w") as f:
+        json.dump(job, f)
+    filled = capture_profile.fill_job(cfg, os.path.join(work, "profiles"),
+                                      os.path.join(work, "filled.json"), quiet=True)
+    hp_kernels = filled[-1].get("additional_num_kernels", filled[-1]["num_kernels"])
+    co_dir = os.path.join(work, "co")
+    co = colocate.run_job(copy.deepcopy(filled), "orion", co_dir, 400000,
+                          env={"ORION_RECORD_DIR": co_dir}, hp_limit=12,
+                          start_update=int(hp_kernels * 0.9))
+    assert co[-1]["iterations"] == 45 and co[0]["iterations"] >= 10
+    assert co[-1]["final_loss"] == co[-1]["final_loss"]          # not NaN
+    dec = _check_replay(co_dir)
+    # every high-priority record was handed to the scheduler thread's own stream
+    assert sum(1 for l in dec.splitlines() if l.startswith("D 1 1 k")) >= 45 * hp_kernels - hp_kernels
