@@ -94,8 +94,12 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     const int super = seq / 32;        // 32 tiles of every super-tile per XCD
     const int local = seq % 32;
     const int supers_n = tiles_n / kSuper;
-    *tm = (super / supers_n) * kSuper + (xcd / 2) * 4 + local % 4;
-    *tn = (super % supers_n) * kSuper + (xcd % 2) * 8 + local / 4;
+    // super-tiles in boustrophedon order: consecutive rounds share their A or
+    // their B panels, which the memory-side cache still holds
+    const int sr = super / supers_n;
+    const int sc = (sr & 1) ? supers_n - 1 - super % supers_n : super % supers_n;
+    *tm = sr * kSuper + (xcd / 2) * 4 + local % 4;
+    *tn = sc * kSuper + (xcd % 2) * 8 + local / 4;
     return;
   }
   int lid = bid;
