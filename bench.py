@@ -21,7 +21,6 @@ the GPU when it starts them):
 """
 
 import argparse
-import copy
 import json
 import os
 import sys

@@ -18,7 +18,6 @@ import json
 import os
 import subprocess
 import sys
-import threading
 
 import torch
 

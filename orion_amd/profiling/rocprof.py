@@ -178,7 +178,6 @@ def collect(config, client, rocprof_dir, iters=12, timeout=300):
     """Run the four rocprofv3 passes over the standalone client.  The caller
     must not have touched the GPU (the profiler starts a fresh process)."""
     import subprocess
-    import sys
     pkg_root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     env = dict(os.environ, TMPDIR="/tmp")
     env["PYTHONPATH"] = pkg_root + (":" + env["PYTHONPATH"] if env.get("PYTHONPATH") else "")

@@ -9,7 +9,6 @@ ten warm-up iterations, measured run -- with the same rendezvous points on
 the library object, scheduler_frontend.py:56, which has no effect).
 """
 
-import ctypes
 from ctypes import (POINTER, c_bool, c_char_p, c_float, c_int, c_void_p)
 import time
 

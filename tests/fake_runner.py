@@ -20,7 +20,7 @@ os.environ["ORION_HIP_LIBRARY"] = os.path.join(ROOT, "tests", "fakehip", "libfak
 
 import numpy as np  # noqa: E402
 
-from orion_amd import _lib, scheduler_frontend as fe  # noqa: E402
+from orion_amd import scheduler_frontend as fe  # noqa: E402
 
 workdir, algo, n_be, hp_iters = sys.argv[1], sys.argv[2], int(sys.argv[3]), int(sys.argv[4])
 hp_graph = len(sys.argv) > 5 and sys.argv[5] == "graph"

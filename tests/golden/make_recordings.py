@@ -15,7 +15,6 @@ tests/test_golden_recordings.py replays every one of them with the CPU oracle an
 with the native policy core and expects the recorded decisions, byte for byte.
 """
 
-import glob
 import os
 import shutil
 import subprocess

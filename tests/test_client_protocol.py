@@ -4,7 +4,6 @@ Pinned by closed forms and by the reference's own job files and arrival trace
 read in place (reference: benchmarking/benchmark_suite/train_imagenet.py:71-241,
 benchmarking/launch_jobs.py:44-148, src/scheduler_frontend.py:17-94)."""
 
-import ctypes
 import glob
 import json
 import os

@@ -8,7 +8,6 @@ scripted traces also run through the native core, so a mistake common to both
 restatements (a dropped term, a wrong index) fails here.
 """
 
-import ctypes
 
 import numpy as np
 import pytest
