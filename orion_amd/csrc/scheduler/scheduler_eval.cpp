@@ -388,13 +388,21 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
   const HipApi* hip = orion_hip_api();
   const pid_t mytid = (pid_t)syscall(SYS_gettid);
 
+  // CUs of the device: what streams and CU masks are built from.
   int cus = 0;
-  if (const char* e = getenv("ORION_MAX_SMS")) cus = atoi(e);
-  if (cus <= 0) {
+  {
     int dev = 0;
     if (hip->hipGetDevice) (void)hip->hipGetDevice(&dev);
     check(hip->hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
           "hipDeviceGetAttribute(MultiprocessorCount)");
+  }
+  // The policy's max_sms (the reference hard-codes 80, its GPU's SM count,
+  // scheduler_eval.cpp:9): the CU budget best-effort kernels may add up to while
+  // a high-priority inference request is in flight.  The device's CU count
+  // unless ORION_MAX_SMS names a smaller budget.
+  int max_sms = cus;
+  if (const char* e = getenv("ORION_MAX_SMS")) {
+    if (atoi(e) > 0) max_sms = atoi(e);
   }
   g.total_cus = cus;
   g.masks = parse_int_list(getenv("ORION_BE_CU_MASKS"));
@@ -429,7 +437,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
   // budget off the whole-GPU stream even while the high-priority client is idle.
   const bool confine_long = getenv("ORION_CONFINE_LONG_BE") &&
                             atoi(getenv("ORION_CONFINE_LONG_BE")) != 0;
-  g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, cus, g.masks,
+  g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, max_sms, g.masks,
                             !as_written, confine_long));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
   g.host->set_policy(g.policy.get());
@@ -439,7 +447,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
     if (*dir) {
       g.record_dir = dir;
       g.recorder.reset(new Recorder(g.host.get(), num_clients));
-      g.recorder->header(cus, g.masks, confine_long);
+      g.recorder->header(max_sms, g.masks, confine_long);
       for (int i = 0; i < num_clients; ++i)
         g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
       // start both logs afresh
