@@ -7,7 +7,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-REFERENCE = "/root/reference"
+REFERENCE = os.environ.get("ORION_REFERENCE_DIR", "/root/reference")
 
 
 def pytest_configure(config):
