@@ -58,7 +58,8 @@ def _c3_job(hp_iters):
     ]
 
 
-def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_graph=False):
+def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_graph=False,
+               repeats=1):
     from orion_amd import colocate
     from orion_amd.profiling import capture_profile
     os.makedirs(workdir, exist_ok=True)
@@ -72,7 +73,7 @@ def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_gr
     if masks:
         env["ORION_BE_CU_MASKS"] = masks
     os.makedirs(env["ORION_RECORD_DIR"], exist_ok=True)
-    res = colocate.experiment(job, "orion", max_be_duration, workdir, env=env)
+    res = colocate.experiment(job, "orion", max_be_duration, workdir, env=env, repeats=repeats)
     res["num_kernels"] = {"hp": job[-1]["num_kernels"],
                           "be": job[0].get("additional_num_kernels", job[0]["num_kernels"])}
     return res
@@ -155,6 +156,10 @@ def main():
                     help="skip the extra run with a HIP-graph high-priority client")
     ap.add_argument("--pair-requests", type=int, default=300,
                     help="measured GEMM requests of the scheduled kernel pair")
+    ap.add_argument("--repeats", type=int, default=3,
+                    help="the isolated and the co-located run of the high-priority client "
+                         "alternate this many times, --steps / --repeats requests each, and "
+                         "the percentiles are taken over all of them")
     ap.add_argument("--workdir", default="")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -172,14 +177,22 @@ def main():
                       "algo": "orion", "max_be_duration_ns": args.max_be_duration}}
     if not args.kernels_only:
         t0 = time.time()
-        co = colocation(args.steps, workdir, args.max_be_duration, args.be_cu_masks,
-                        args.rocprof_profiles)
+        repeats = max(1, args.repeats)
+        co = colocation(-(-args.steps // repeats), workdir, args.max_be_duration,
+                        args.be_cu_masks, args.rocprof_profiles, repeats=repeats)
         out["value"] = co["hp_p99_ratio"]
         out["ms_per_step"] = 1000.0 / co["hp_colocated"]["throughput"]
         out["hp"] = {"isolated_ms": {k: co["hp_isolated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
                      "colocated_ms": {k: co["hp_colocated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
                      "p50_ratio": co["hp_p50_ratio"], "p99_ratio": co["hp_p99_ratio"],
-                     "requests_per_s": co["hp_colocated"]["throughput"]}
+                     "requests_per_s": co["hp_colocated"]["throughput"],
+                     # the alternating runs one by one (percentiles above: all requests)
+                     "isolated_runs_p99_ms": [r["p99_latency"] for r in
+                                              co["hp_isolated"].get("runs", [])],
+                     "colocated_runs_p99_ms": [r["p99_latency"] for r in
+                                               co["hp_colocated"].get("runs", [])],
+                     "requests": {"isolated": co["hp_isolated"].get("requests"),
+                                  "colocated": co["hp_colocated"].get("requests")}}
         out["be"] = {"isolated_iters_per_s": co["be_isolated"][0]["throughput"],
                      "colocated_iters_per_s": co["be_colocated"][0]["throughput"],
                      "retained": co["be_retained"][0]}

@@ -196,5 +196,9 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
     if extra:
         data.update(extra())
     data["iterations"] = batch_idx
+    if not train:
+        # every measured request, in arrival order (the reference's file holds
+        # the percentiles only): lets runs be pooled
+        data["latencies_ms"] = [round(t * 1000, 4) for t in timings[drop:]]
     write_result(tid, data)
     return data

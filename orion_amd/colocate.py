@@ -17,6 +17,8 @@ import subprocess
 import sys
 import tempfile
 
+import numpy as np
+
 from . import _lib
 
 
@@ -63,15 +65,40 @@ def run_job(job, algo, workdir, max_be_duration, reef_depth=12, env=None,
     return out
 
 
+def pooled(runs):
+    """One result for a client measured in several runs: latency percentiles
+    over all runs' requests together, throughput averaged."""
+    out = {"throughput": sum(r["throughput"] for r in runs) / len(runs)}
+    lat = [t for r in runs for t in r.get("latencies_ms", [])]
+    if lat and all("latencies_ms" in r for r in runs):
+        for p in (50, 95, 99):
+            out[f"p{p}_latency"] = float(np.percentile(lat, p))
+        out["requests"] = len(lat)
+    elif "p99_latency" in runs[0]:
+        assert len(runs) == 1
+        out.update({k: runs[0][k] for k in ("p50_latency", "p95_latency", "p99_latency")})
+    if len(runs) > 1:
+        out["runs"] = [{k: r[k] for k in ("p50_latency", "p95_latency", "p99_latency",
+                                          "throughput") if k in r} for r in runs]
+    return out
+
+
 def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
-               be_isolated_iters=60, env=None, skip_isolated=False):
+               be_isolated_iters=60, env=None, skip_isolated=False, repeats=1):
+    """Runs the high-priority client alone, every best-effort client alone, and
+    the whole job; reports the high-priority client's latency ratios and what
+    each best-effort client keeps of its own throughput.
+
+    With ``repeats`` > 1 the isolated and the co-located run of the high-priority
+    client alternate that many times and their requests are pooled: the speed of
+    one run drifts by 10-20 % on the same machine (clock and power state), which
+    is as large as the effect being measured."""
     workdir = workdir or tempfile.mkdtemp(prefix="orion_colocate_")
     hp = job[-1]
     result = {"algo": algo, "max_be_duration_ns": max_be_duration, "workdir": workdir}
+    env = dict(env or {})
+    record_dir = env.pop("ORION_RECORD_DIR", None)
     if not skip_isolated:
-        iso_hp = run_job([copy.deepcopy(hp)], algo, os.path.join(workdir, "iso_hp"),
-                         max_be_duration, env=env)[0]
-        result["hp_isolated"] = iso_hp
         result["be_isolated"] = []
         for k, be in enumerate(job[:-1]):
             entry = copy.deepcopy(be)
@@ -79,22 +106,36 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
             result["be_isolated"].append(
                 run_job([entry], algo, os.path.join(workdir, f"iso_be{k}"),
                         max_be_duration, env=env)[0])
-    if len(job) > 1:
-        co = run_job(copy.deepcopy(job), algo, os.path.join(workdir, "colocated"),
-                     max_be_duration, env=env)
-        result["hp_colocated"] = co[-1]
-        result["be_colocated"] = co[:-1]
+    iso_runs, co_runs = [], []
+    for rep in range(repeats):
+        tag = f"_{rep}" if repeats > 1 else ""
         if not skip_isolated:
-            if "p99_latency" in co[-1] and "p99_latency" in result["hp_isolated"]:
+            iso_runs.append(run_job([copy.deepcopy(hp)], algo,
+                                    os.path.join(workdir, "iso_hp" + tag),
+                                    max_be_duration, env=env)[0])
+        if len(job) > 1:
+            co_env = dict(env)
+            if record_dir and rep == repeats - 1:      # the last run keeps the logs
+                co_env["ORION_RECORD_DIR"] = record_dir
+            co_runs.append(run_job(copy.deepcopy(job), algo,
+                                   os.path.join(workdir, "colocated" + tag),
+                                   max_be_duration, env=co_env))
+    if iso_runs:
+        result["hp_isolated"] = pooled(iso_runs)
+    if co_runs:
+        result["hp_colocated"] = pooled([co[-1] for co in co_runs])
+        result["be_colocated"] = [pooled([co[k] for co in co_runs])
+                                  for k in range(len(job) - 1)]
+        if iso_runs:
+            iso, co_hp = result["hp_isolated"], result["hp_colocated"]
+            if "p99_latency" in co_hp and "p99_latency" in iso:
                 for p in ("p50", "p95", "p99"):
-                    result[f"hp_{p}_ratio"] = (co[-1][f"{p}_latency"]
-                                               / result["hp_isolated"][f"{p}_latency"])
+                    result[f"hp_{p}_ratio"] = co_hp[f"{p}_latency"] / iso[f"{p}_latency"]
             else:
-                result["hp_throughput_retained"] = (
-                    co[-1]["throughput"] / result["hp_isolated"]["throughput"])
+                result["hp_throughput_retained"] = co_hp["throughput"] / iso["throughput"]
             result["be_retained"] = [
                 c["throughput"] / i["throughput"] if i["throughput"] > 0 else 0.0
-                for c, i in zip(co[:-1], result["be_isolated"])]
+                for c, i in zip(result["be_colocated"], result["be_isolated"])]
     return result
 
 

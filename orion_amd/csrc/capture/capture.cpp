@@ -43,11 +43,59 @@ inline void cpu_relax(unsigned& spins) {
   if ((++spins & 0x3ff) == 0) sched_yield();
 }
 
+// Thread placement (reference: utils_interc.cpp:36-49 pins client idx, and the
+// scheduler as idx N, to CPU idx + 1 the first time it is identified).  Here
+// slot s is the (s + 1)-th CPU the process may run on, the first one staying
+// with the interpreter's other threads; the masks in force before are put back
+// when the capture is disarmed.  ORION_PIN_THREADS=0 leaves placement to the
+// kernel, as does a CPU set too small for one CPU per slot.
+struct Pinning {
+  bool on = false;
+  int cpus[kMaxClients + 2];
+  pid_t tid[kMaxClients + 1];
+  cpu_set_t before[kMaxClients + 1];
+};
+Pinning g_pin;
+
+void pinning_reset(int slots) {
+  for (pid_t& t : g_pin.tid) t = 0;
+  const char* env = getenv("ORION_PIN_THREADS");
+  g_pin.on = false;
+  if (env && atoi(env) == 0) return;
+  cpu_set_t allowed;
+  if (sched_getaffinity(getpid(), sizeof allowed, &allowed) != 0) return;
+  int n = 0;
+  for (int c = 0; c < CPU_SETSIZE && n < slots + 1; ++c)
+    if (CPU_ISSET(c, &allowed)) g_pin.cpus[n++] = c;
+  g_pin.on = n == slots + 1;
+}
+
+void pin_caller(int slot, pid_t tid) {
+  if (!g_pin.on || g_pin.tid[slot] == tid) return;
+  if (sched_getaffinity(0, sizeof(cpu_set_t), &g_pin.before[slot]) != 0) return;
+  cpu_set_t one;
+  CPU_ZERO(&one);
+  CPU_SET(g_pin.cpus[slot + 1], &one);
+  if (sched_setaffinity(0, sizeof one, &one) == 0) g_pin.tid[slot] = tid;
+}
+
+void pinning_undo() {
+  for (int s = 0; s <= kMaxClients; ++s) {
+    if (g_pin.tid[s] == 0) continue;
+    // a thread that has ended leaves ESRCH, which is fine
+    (void)sched_setaffinity(g_pin.tid[s], sizeof(cpu_set_t), &g_pin.before[s]);
+    g_pin.tid[s] = 0;
+  }
+}
+
 int lookup_thread() {
   const pid_t tid = (pid_t)syscall(SYS_gettid);
   if (tid == g_state.scheduler_tid) return kNotClient;
   for (int i = 0; i < g_state.num_clients; ++i)
-    if (g_state.client_tids[i] == tid) return i;
+    if (g_state.client_tids[i] == tid) {
+      pin_caller(i, tid);
+      return i;
+    }
   return kNotClient;
 }
 
@@ -212,8 +260,11 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
     abort();
   }
   g_state.armed.store(0, std::memory_order_release);
+  pinning_undo();
+  pinning_reset(num_clients + 1);
   g_state.num_clients = num_clients;
   g_state.scheduler_tid = scheduler_tid;
+  if ((pid_t)syscall(SYS_gettid) == scheduler_tid) pin_caller(num_clients, scheduler_tid);
   for (int i = 0; i < num_clients; ++i) {
     g_state.client_tids[i] = client_tids ? client_tids[i] : 0;
     ClientChannel& ch = g_state.channels[i];
@@ -236,6 +287,15 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
 void orion_capture_disarm(void) {
   g_state.armed.store(0, std::memory_order_release);
   g_state.epoch.fetch_add(1, std::memory_order_acq_rel);
+  pinning_undo();
+}
+
+// The CPU the capture pinned the calling thread to, or -1.
+int orion_pinned_cpu(void) {
+  const pid_t tid = (pid_t)syscall(SYS_gettid);
+  for (int s = 0; s <= kMaxClients; ++s)
+    if (g_pin.tid[s] == tid) return g_pin.cpus[s + 1];
+  return -1;
 }
 
 // Registers the calling thread as a thread of `client` (alternative to passing

@@ -78,6 +78,7 @@ for c in range(n_clients):
     files.append(p)
 
 results = [None] * n_clients
+placement = [None] * (n_clients + 1)     # (pinned cpu, allowed set) while the job runs
 iters_done = [0] * n_clients
 barriers = [threading.Barrier(n_clients + 1)]
 
@@ -125,6 +126,10 @@ def client(tid):
         cap.block(it)
         it += 1
         iters_done[tid] = it
+        if it == 1:
+            placement[tid] = (cap.orion_pinned_cpu(), sorted(os.sched_getaffinity(0)))
+            if tid == n_clients - 1:      # the scheduler thread, seen from outside
+                placement[n_clients] = sorted(os.sched_getaffinity(sched_tid[0]))
         if it in (1, 10):
             barriers[0].wait()
         if cap.stop():
@@ -155,6 +160,7 @@ for t in threads:
 tids = [t.native_id for t in threads]
 py = fe.PyScheduler(sched, n_clients)
 sched_tid = []
+sched_after = []
 
 
 def run_sched():
@@ -163,6 +169,7 @@ def run_sched():
                      [None] * n_clients, records_per_iter, [None] * n_clients,
                      iters, True, True, algo == "reef", algo == "sequential",
                      8 if algo == "reef" else 100_000, 1, 1, [True] * n_be + [False])
+    sched_after.extend(sorted(os.sched_getaffinity(0)))
 
 
 st = threading.Thread(target=run_sched)
@@ -190,6 +197,8 @@ for c in range(n_clients):
 
 print(json.dumps({
     "alive": alive, "iters_done": iters_done, "outputs_equal": ok_outputs,
+    "placement": placement[:n_clients], "scheduler_placement": placement[n_clients],
+    "scheduler_mask_after": sched_after, "allowed_cpus": sorted(os.sched_getaffinity(0)),
     "launch_tids": launch_tids, "sched_tid": sched_tid, "client_tids": tids,
     "launch_stream_masks": masks, "n_launches": sum(1 for k, s, t in log if k == 0),
     "launch_streams_by_tid": {str(t): sorted({s for k, s, tt in log if k == 0 and tt == t})

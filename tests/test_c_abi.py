@@ -20,7 +20,7 @@ def declared(header):
 
 
 CAPTURE_SYMBOLS = {"block", "stop", "orion_register_thread", "orion_register_stream",
-                   "orion_client_index", "orion_client_of_stream",
+                   "orion_client_index", "orion_client_of_stream", "orion_pinned_cpu",
                    "orion_thread_passthrough"}
 
 

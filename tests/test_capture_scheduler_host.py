@@ -33,14 +33,15 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FAKEHIP = os.path.join(ROOT, "tests", "fakehip", "libfakehip.so")
 
 
-def run_child(workdir, algo, n_be, hp_iters, direct=True, graph=False):
+def run_child(workdir, algo, n_be, hp_iters, direct=True, graph=False, pin=True):
     if not os.path.exists(FAKEHIP):
         pytest.fail("tests/fakehip/libfakehip.so is not built (make -C orion_amd/csrc)")
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), workdir,
          algo, str(n_be), str(hp_iters)] + (["graph"] if graph else []),
         capture_output=True, text=True, timeout=300,
-        env=dict(os.environ, ORION_HP_DIRECT="1" if direct else "0"))
+        env=dict(os.environ, ORION_HP_DIRECT="1" if direct else "0",
+                 ORION_PIN_THREADS="1" if pin else "0"))
     assert proc.returncode == 0, proc.stdout + proc.stderr
     line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
     return json.loads(line)
@@ -99,6 +100,29 @@ def test_a_captured_graph_is_one_record(tmp_path, direct):
     hp = [l.split() for l in dec.splitlines() if l.startswith(f"D 2 ")]
     assert sum(1 for x in hp if x[3] == "k") == hp_iters      # one kernel record each
     assert obslog.replay(obs) == dec and jobs.native_replay(obs) == dec
+
+
+@pytest.mark.parametrize("pin", [True, False])
+def test_client_threads_are_pinned_while_the_job_runs(tmp_path, pin):
+    """reference: utils_interc.cpp:36-49 -- each client thread gets a CPU of its
+    own the first time it is identified.  Client i runs on the (i + 2)-th CPU
+    the process may use (the first stays with the other threads); the mask is
+    given back when the job ends; ORION_PIN_THREADS=0 pins nothing."""
+    n_be = 2
+    if len(os.sched_getaffinity(0)) < n_be + 3:
+        pytest.skip("fewer CPUs than clients + scheduler + 1")
+    res = run_child(str(tmp_path), "orion", n_be, 20, pin=pin)
+    assert not any(res["alive"]) and all(res["outputs_equal"])
+    allowed = res["allowed_cpus"]            # main thread, after the job: untouched
+    assert allowed == sorted(os.sched_getaffinity(0))
+    for i, (cpu, mask) in enumerate(res["placement"]):
+        if pin:
+            assert cpu == allowed[i + 1] and mask == [cpu]
+        else:
+            assert cpu == -1 and mask == allowed
+    # the scheduler thread takes the slot after the last client
+    assert res["scheduler_placement"] == ([allowed[n_be + 2]] if pin else allowed)
+    assert res["scheduler_mask_after"] == allowed
 
 
 def test_kernel_count_mismatch_ends_the_job_with_a_report(tmp_path):

@@ -159,3 +159,22 @@ def test_frontend_rejects_mismatched_lists():
         py.run_scheduler([threading.Barrier(1)], [1, 2], ["a", "b"], ["f", "g"], [None, None],
                          [1, 1], [None, None], [1, 1], True, False, False, False, 1, 1, 1,
                          [False, False])
+
+
+def test_repeated_runs_are_pooled_request_by_request():
+    """colocate.pooled: percentiles over all runs' requests together (not a mean
+    of per-run percentiles), throughput averaged, the runs kept one by one."""
+    from orion_amd import colocate
+    a = {"throughput": 80.0, "p50_latency": 1.0, "p95_latency": 1.0, "p99_latency": 1.0,
+         "latencies_ms": [1.0] * 99 + [50.0]}
+    b = {"throughput": 60.0, "p50_latency": 3.0, "p95_latency": 3.0, "p99_latency": 3.0,
+         "latencies_ms": [3.0] * 100}
+    res = colocate.pooled([a, b])
+    want = np.percentile([1.0] * 99 + [50.0] + [3.0] * 100, [50, 95, 99])
+    assert [res["p50_latency"], res["p95_latency"], res["p99_latency"]] == list(want)
+    assert res["throughput"] == 70.0 and res["requests"] == 200 and len(res["runs"]) == 2
+    # a training client has no latencies: throughput only
+    assert colocate.pooled([{"throughput": 30.0}, {"throughput": 34.0}])["throughput"] == 32.0
+    # one run without the raw list (an older result file) keeps its own percentiles
+    old = {k: v for k, v in a.items() if k != "latencies_ms"}
+    assert colocate.pooled([old])["p99_latency"] == 1.0
