@@ -26,6 +26,7 @@ def _function_dict():
     # imported lazily: the model code needs torch, the argument parser does not
     from .benchmark_suite.bert_trainer import bert_loop
     from .benchmark_suite.train_imagenet import imagenet_loop
+    from .benchmark_suite.transformer_trainer import transformer_loop
     from .kernel_pair import gemm_loop, triad_loop
     return {
         "gemm_bf16": gemm_loop,
@@ -34,6 +35,7 @@ def _function_dict():
         "resnet101": imagenet_loop,
         "mobilenet_v2": imagenet_loop,
         "bert": bert_loop,
+        "transformer": transformer_loop,
     }
 
 

@@ -180,6 +180,58 @@ def test_mobilenet_beside_bert_training(tmp_path):
     _check_replay(co_dir)
 
 
+def test_transformer_xl_trainer_beside_mobilenet(tmp_path):
+    """The reference's fig7/config_files/trans_mnet.json: a Transformer-XL
+    trainer (relative attention, adaptive softmax with its device-to-host
+    reads, LAMB) as the best-effort client."""
+    job = [
+        {"arch": "transformer", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
+         "args": {"batchsize": 2, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": True, "dtype": "fp32"}},
+        {"arch": "mobilenet_v2", "kernel_file": "", "num_kernels": 0, "num_iters": 40,
+         "args": {"model_name": "mobilenet_v2", "batchsize": 4, "rps": 0, "uniform": False,
+                  "dummy_data": True, "train": False, "dtype": "fp32"}},
+    ]
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job, 100000)
+    assert co[-1]["iterations"] == 40 and co[0]["iterations"] >= 10
+    assert filled[0]["num_kernels"] > 500
+    ref = _mobilenet_cpu_reference(4)
+    for out in (iso_out, co_out):
+        assert float((out - ref).abs().max() / ref.abs().max()) <= CPU_RTOL
+    _check_replay(co_dir)
+
+
+def test_transformer_xl_inference_client(tmp_path):
+    """Transformer-XL inference as the high-priority client beside the triad
+    loop: the per-token losses of the last request -- which depend on the memory
+    every earlier request left -- against the same steps on the PyTorch CPU path."""
+    from orion_amd.benchmark_suite import client_common as cc
+    from orion_amd.benchmark_suite import transformer_trainer as tt
+    n_req, small = 12, {"n_layer": 4}
+    job = [
+        {"arch": "triad_f32", "kernel_file": "", "num_kernels": 0, "num_iters": 1_000_000,
+         "args": {"batchsize": 1 << 22, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": True}},
+        {"arch": "transformer", "kernel_file": "", "num_kernels": 0, "num_iters": n_req,
+         "args": {"batchsize": 2, "rps": 0, "uniform": False, "dummy_data": True,
+                  "train": False, "dtype": "fp32", "model_config": small}},
+    ]
+    filled, co, iso_out, co_out, co_dir = _run_iso_and_co(str(tmp_path), job)
+    assert co[-1]["iterations"] == n_req
+    assert torch.equal(iso_out, co_out)
+    with cc.MODEL_INIT_LOCK:
+        cc.seed_everything(42)
+        model = tt.MemTransformerLM(**dict(tt.MODEL_CONFIG, **small)).eval()
+    data, target = tt.DummyDataLoader(2, 42).batch()
+    mems = None
+    with torch.no_grad():
+        for _ in range(cc.UNCAPTURED_STEPS + n_req):
+            ref, mems = model(data, target, mems)
+    assert co_out.shape == ref.shape == (192, 2)
+    assert float((co_out - ref).abs().max() / ref.abs().max()) <= CPU_RTOL
+    _check_replay(co_dir)
+
+
 def test_four_clients_round_robin(tmp_path):
     """N = 4 (reference: multi_client_example.json; round-robin over the
     best-effort clients, scheduler_eval.cpp:323-326): a model client with three
