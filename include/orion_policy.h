@@ -28,6 +28,12 @@ extern "C" {
  * client is past its tenth iteration). */
 int orion_policy_replay(const char* observations, int sequential_fix,
                         char** decisions_out, char** error_out);
+/* The same replay; the decision log carries a line "P" before the decisions
+ * of every logged poll, so that decisions can be read poll by poll beside the
+ * observation log's P lines (one iteration of the loop at
+ * scheduler_eval.cpp:277-302 each). */
+int orion_policy_replay_by_poll(const char* observations, int sequential_fix,
+                                char** decisions_out, char** error_out);
 void orion_policy_free(char* p);
 
 /* populate_kernel_info + the max-SM scan of setup (scheduler_eval.cpp:498-526,

@@ -86,6 +86,7 @@ class RecordingEnv(po.Env):
         self.algo = algo
         self.budget = None            # Orion's best-effort duration budget (ns)
         self.confine_long = False     # placement option, header token L1
+        self.mark_polls = False       # a "P" line before every poll's decisions
         self.obs = []
         self.dec = DecisionLog()
         self._reset_poll()
@@ -132,6 +133,8 @@ class RecordingEnv(po.Env):
             ev = "".join("1" if e else "0" for e in self._events) or "-"
             us = ",".join(str(u) for u in self._us) or "-"
             self.obs.append(f"P {acks:x} {''.join(self._heads)} {ev} {us}")
+            if self.mark_polls:
+                self.dec.add("P")
             for line in self._dec:
                 self.dec.add(line)
         else:
@@ -241,8 +244,9 @@ class ReplayEnv(po.Env):
         pass
 
 
-def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
-    """Run the oracle over an observation log; return its decision log text."""
+def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_polls=False):
+    """Run the oracle over an observation log; return its decision log text
+    (with ``mark_polls``, a line ``P`` precedes every logged poll's decisions)."""
     oracle = None
     rec = None
     n = max_sms = masks = None
@@ -289,6 +293,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True):
                                    lambda c, k: oracle.ops[c][k],
                                    hp_active=lambda: oracle.seen[n - 1] > 0)
             rec.inner = env
+            rec.mark_polls = mark_polls
             warmup, witers, algo = bool(int(parts[1])), int(parts[2]), parts[3]
             depth, hp_limit, ustart = int(parts[4]), int(parts[5]), int(parts[6])
             rec.algo = algo

@@ -74,6 +74,7 @@ void Recorder::end_poll(bool effective) {
     obs_ += ' ';
     obs_ += us_.empty() ? "-" : us_;
     obs_ += '\n';
+    if (mark_polls_) dec_ += "P\n";
     dec_ += poll_dec_;
   }
   inner_->end_poll(effective);
@@ -209,7 +210,7 @@ struct ClientDesc { int nk = 0, ni = 0; bool train = false; std::string path; bo
 }  // namespace
 
 bool replay_observations(const std::string& obs, bool sequential_fix,
-                         std::string* decisions, std::string* err) {
+                         std::string* decisions, std::string* err, bool mark_polls) {
   std::vector<std::string> lines;
   {
     size_t at = 0;
@@ -256,6 +257,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
       if (n < 1 || n > 64) { ok = bad(i, "client count out of range"); break; }
       clients.assign((size_t)n, ClientDesc());
       rec = Recorder(&idle, n);
+      rec.set_mark_polls(mark_polls);
     } else if (tag == 'K') {
       auto p = split(l, ' ', 6);
       if (p.size() != 6) { ok = bad(i, "K needs 5 fields"); break; }

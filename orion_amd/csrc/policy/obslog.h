@@ -34,6 +34,9 @@ class Recorder : public PolicyHost {
  public:
   Recorder(PolicyHost* inner, int n) : inner_(inner), n_(n) {}
   void set_inner(PolicyHost* inner) { inner_ = inner; }
+  // With marks, a line "P" precedes the decisions of every effective poll, so
+  // the decision log lines up with the observation log's P lines one to one.
+  void set_mark_polls(bool on) { mark_polls_ = on; }
 
   void header(int max_sms, const std::vector<int>& masks, bool confine_long = false);
   void client(int idx, int num_kernels, int num_iters, bool train,
@@ -59,6 +62,7 @@ class Recorder : public PolicyHost {
  private:
   PolicyHost* inner_;
   int n_;
+  bool mark_polls_ = false;
   std::string obs_, dec_;
   // current poll
   unsigned long long acks_ = 0;
@@ -68,6 +72,7 @@ class Recorder : public PolicyHost {
 // Replays an observation log through the native policy; returns false and
 // fills *err when the log is malformed or the policy diverges from it.
 bool replay_observations(const std::string& obs, bool sequential_fix,
-                         std::string* decisions, std::string* err);
+                         std::string* decisions, std::string* err,
+                         bool mark_polls = false);
 
 }  // namespace orion

@@ -18,19 +18,30 @@ char* dup_string(const std::string& s) {
 
 extern "C" {
 
-int orion_policy_replay(const char* observations, int sequential_fix,
-                        char** decisions_out, char** error_out) {
+static int replay(const char* observations, int sequential_fix, bool mark_polls,
+                  char** decisions_out, char** error_out) {
   if (decisions_out) *decisions_out = nullptr;
   if (error_out) *error_out = nullptr;
   if (!observations) return 1;
   std::string dec, err;
-  bool ok = orion::replay_observations(observations, sequential_fix != 0, &dec, &err);
+  bool ok = orion::replay_observations(observations, sequential_fix != 0, &dec, &err,
+                                       mark_polls);
   if (!ok) {
     if (error_out) *error_out = dup_string(err);
     return 2;
   }
   if (decisions_out) *decisions_out = dup_string(dec);
   return 0;
+}
+
+int orion_policy_replay(const char* observations, int sequential_fix,
+                        char** decisions_out, char** error_out) {
+  return replay(observations, sequential_fix, false, decisions_out, error_out);
+}
+
+int orion_policy_replay_by_poll(const char* observations, int sequential_fix,
+                                char** decisions_out, char** error_out) {
+  return replay(observations, sequential_fix, true, decisions_out, error_out);
 }
 
 void orion_policy_free(char* p) { free(p); }

@@ -138,6 +138,8 @@ def policy_lib():
             ctypes.c_char_p, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
             ctypes.POINTER(ctypes.c_void_p)]
         lib.orion_policy_replay.restype = ctypes.c_int
+        lib.orion_policy_replay_by_poll.argtypes = lib.orion_policy_replay.argtypes
+        lib.orion_policy_replay_by_poll.restype = ctypes.c_int
         lib.orion_policy_free.argtypes = [ctypes.c_void_p]
         lib.orion_policy_free.restype = None
         lib.orion_profile_stats.argtypes = [
@@ -155,12 +157,12 @@ def policy_lib():
     return _policy
 
 
-def native_replay(obs_text, sequential_fix=True):
+def native_replay(obs_text, sequential_fix=True, by_poll=False):
     """Decision log of the native policy core for an observation log."""
     lib = policy_lib()
     out, err = ctypes.c_void_p(), ctypes.c_void_p()
-    rc = lib.orion_policy_replay(obs_text.encode(), int(sequential_fix),
-                                 ctypes.byref(out), ctypes.byref(err))
+    fn = lib.orion_policy_replay_by_poll if by_poll else lib.orion_policy_replay
+    rc = fn(obs_text.encode(), int(sequential_fix), ctypes.byref(out), ctypes.byref(err))
     try:
         if rc != 0:
             msg = ctypes.string_at(err).decode() if err else f"rc={rc}"

@@ -35,7 +35,7 @@ def test_kernels_header():
 
 def test_policy_header():
     names = declared("orion_policy.h")
-    assert "orion_policy_replay" in names and len(names) == 5
+    assert "orion_policy_replay" in names and "orion_policy_replay_by_poll" in names and len(names) == 6
     lib = _lib.load(_lib.POLICY_LIB)
     for n in names:
         assert hasattr(lib, n)

@@ -31,6 +31,14 @@ def _check_replay(record_dir):
     assert dec.count("\nD ") > 50
     assert jobs.native_replay(obs) == dec
     assert obslog.replay(obs) == dec
+    # the reference's per-poll rules, on this live run (Orion, inference HP)
+    lines = obs.splitlines()
+    n = int(lines[0].split(" ")[1])
+    hp_trains = next(l for l in lines if l.startswith(f"K {n - 1} ")).split(" ")[4] == "1"
+    seg = next(l for l in lines if l.startswith("S ")).split(" ")
+    if seg[3] == "orion" and not hp_trains:
+        from tests.test_policy_properties import check_orion_invariants
+        check_orion_invariants(obs, jobs.native_replay(obs, by_poll=True), int(seg[4]))
     return dec
 
 

@@ -1,0 +1,205 @@
+"""Invariants of the Orion policy, checked poll by poll on the NATIVE core.
+
+hypothesis draws jobs (profiles, traces, arrival patterns, budgets, client
+counts); the virtual-time model produces an observation log; the native core
+replays it with poll marks (orion_policy_replay_by_poll).  The checks below are
+read off the reference's loop (src/scheduler/scheduler_eval.cpp:277-400), not
+off this build's oracle; the only state they keep is the reference's own
+bookkeeping (seen[], iteration counts, the running best-effort duration sum):
+
+* a client whose iteration is fully dispatched is not peeked (:281-282);
+* a high-priority record at the head of its queue is dispatched in the same
+  poll, before any best-effort record (:307-318);
+* one dispatch per client and poll at most, of the record class that was peeked;
+* best-effort clients are visited in rotation from the one after the last
+  client dispatched (:320-323, :383);
+* a best-effort record MUST go out when the high-priority client is idle, the
+  record is a memory operation, the client is within its first ten iterations,
+  or the high-priority client has finished (:330-335) -- unless the duration
+  throttle is on;
+* a best-effort kernel that goes out beside a running high-priority iteration
+  fits the CU budget of this poll and is of the opposite (or unknown) class
+  (:339);
+* once the running sum of profiled durations exceeds the budget nothing
+  best-effort goes out until a poll that queried events (:341-357, :363-367).
+
+Profile durations are whole numbers below 2^24, so the reference's float/long
+sum is exact here.
+"""
+
+import csv
+import os
+
+import pytest
+from hypothesis import HealthCheck, given, settings, strategies as st
+
+from oracle import policy_oracle as po
+from tests import jobs
+
+RECORD = set("kcmfs")
+
+
+def rows_of(path):
+    with open(path) as f:
+        return [(int(r["Profile"]), int(r["SM_usage"]), int(float(r["Duration"])))
+                for r in csv.DictReader(f)]
+
+
+def check_orion_invariants(obs_text, dec_text, depth):
+    obs, dec = obs_text.splitlines(), dec_text.splitlines()
+    at = 0                                   # cursor in dec
+
+    def take(expect=None):
+        nonlocal at
+        line = dec[at]
+        at += 1
+        if expect is not None:
+            assert line == expect, (line, expect)
+        return line
+
+    n = max_sms = None
+    nk, max_iters, prof = {}, {}, {}
+    seen, iters, event_ids = {}, {}, {}
+    checked = {"must": 0, "budget": 0, "throttle": 0, "rotation": 0}
+    for line in obs:
+        p = line.split(" ")
+        if p[0] == "J":
+            n, max_sms = int(p[1]), int(p[2])
+            hp = n - 1
+        elif p[0] == "K":
+            c = int(p[1])
+            nk[c], max_iters[c], prof[c] = int(p[2]), int(p[3]), rows_of(p[5])
+            seen[c], iters[c], event_ids[c] = 0, 0, 0
+        elif p[0] == "X":
+            c = int(p[1])
+            nk[c], prof[c] = int(p[2]), rows_of(p[3])
+            take(f"X {c}")
+        elif p[0] == "S":
+            take("S")
+            throttled, running, start = False, 0, -1      # locals of schedule() (:258-261)
+            hp_profile = None                             # profiles[hp], last HP record's row
+        elif p[0] == "E":
+            take("E")
+        elif p[0] == "P":
+            take("P")
+            heads, events = p[2], p[3]
+            block = []
+            while at < len(dec) and dec[at][0] in "DFT":
+                block.append(take().split(" "))
+            for c in range(n):
+                if seen[c] == nk[c]:
+                    assert heads[c] == "-", (line, c)
+            ds = [b for b in block if b[0] == "D"]
+            clients = [int(b[1]) for b in ds]
+            assert len(set(clients)) == len(clients)
+            for b in ds:
+                assert heads[int(b[1])] == b[3], (line, b)
+            if heads[hp] in RECORD:
+                assert ds and int(ds[0][1]) == hp, (line, block)
+            be_order = [c for c in clients if c != hp]
+            if n > 1 and be_order:
+                rotation = [(start + 1 + i) % (n - 1) for i in range(n - 1)]
+                assert be_order == [c for c in rotation if c in be_order], (start, be_order)
+                checked["rotation"] += 1
+            size = 0
+            poll_throttled = throttled       # on at any moment of this poll
+            for b in ds:
+                c, cls, op = int(b[1]), b[3], int(b[4])
+                assert op == seen[c] and int(b[5]) == event_ids[c]
+                row = prof[c][op] if op < len(prof[c]) else None
+                if c == hp:
+                    hp_profile = row[0] if row else None
+                    if cls == "k":        # only kernel records advance either counter
+                        seen[c] += 1      # (utils_sched.cpp:240-249 against :251-282)
+                        event_ids[c] += 1
+                    continue
+                hp_done = iters[hp] >= max_iters[hp]
+                if throttled:
+                    # released only by a poll that asked the GPU about every
+                    # best-effort client with an event outstanding (:343-352)
+                    if any(event_ids[k] >= 1 for k in range(n - 1)):
+                        assert "1" in events, (line, b)
+                        checked["throttle"] += 1
+                    throttled, running = False, 0
+                free_pass = (n == 1 or seen[hp] == 0 or cls != "k" or iters[c] <= 10
+                             or hp_done)
+                if not free_pass and row is not None and hp_profile is not None:
+                    assert size + row[1] <= max_sms, (line, b, size)
+                    assert row[0] == -1 or hp_profile == -1 or row[0] != hp_profile, (line, b)
+                    checked["budget"] += 1
+                if row is not None:
+                    size += row[1]
+                    if cls == "k":
+                        running += row[2]
+                if cls == "k":
+                    seen[c] += 1
+                    event_ids[c] += 1
+                if running > depth and not hp_done:
+                    throttled = poll_throttled = True
+                start = c
+            # records that had to go out and did not
+            for c in range(n - 1):
+                if heads[c] in RECORD and c not in clients and not poll_throttled:
+                    free_pass = (seen[hp] == 0 or heads[c] != "k" or iters[c] <= 10
+                                 or iters[hp] >= max_iters[hp])
+                    # (a poll during which the throttle was on at any moment does
+                    # not count: on a live GPU the answers of the event queries
+                    # change between two clients of the same rotation)
+                    assert not free_pass, (line, c, block)
+                    checked["must"] += 1
+            for b in block:
+                if b[0] == "F":
+                    c = int(b[1])
+                    assert seen[c] == nk[c] and int(b[2]) == iters[c]
+                    seen[c], iters[c], event_ids[c] = 0, iters[c] + 1, 0
+    assert at == len(dec)
+    return checked
+
+
+@settings(max_examples=150, deadline=None,
+          suppress_health_check=[HealthCheck.function_scoped_fixture, HealthCheck.too_slow])
+@given(seed=st.integers(0, 10_000), n_clients=st.integers(1, 5),
+       depth=st.sampled_from([1, 20_000, 150_000, 600_000, 5_000_000]),
+       hp_iters=st.integers(11, 30))
+def test_orion_invariants_on_the_native_core(tmp_path_factory, seed, n_clients, depth, hp_iters):
+    tmp = str(tmp_path_factory.mktemp("job"))
+    job = jobs.make_job(tmp, seed, n_clients=n_clients, algo=po.ALGO_ORION, hp_train=False,
+                        hp_iters=hp_iters, depth=depth)
+    _, _, rec = jobs.run_oracle(job)
+    obs = rec.obs_text()
+    marked = jobs.native_replay(obs, by_poll=True)
+    assert "".join(l + "\n" for l in marked.splitlines() if l != "P") == rec.dec.text()
+    check_orion_invariants(obs, marked, depth)
+
+
+@pytest.mark.parametrize("case", ["fake_orion_2be", "mi355x_kernel_pair"])
+def test_orion_invariants_on_recordings_of_the_live_scheduler(case):
+    """The same checks on committed recordings of the live native scheduler
+    (the recording HIP stand-in, and the kernel pair on an MI355X)."""
+    d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", case)
+    obs = open(os.path.join(d, "observations.log")).read().replace("@DIR@", d)
+    assert " orion " in obs
+    depth = int(next(l for l in obs.splitlines() if l.startswith("S ")).split(" ")[4])
+    counts = check_orion_invariants(obs, jobs.native_replay(obs, by_poll=True), depth)
+    assert counts["rotation"] > 0
+
+
+def test_the_checks_bite(tmp_path):
+    """The invariants are not vacuous: every kind fires on an ordinary job, and a
+    log with one best-effort dispatch moved to the neighbouring poll fails."""
+    job = jobs.make_job(str(tmp_path), 11, n_clients=3, hp_iters=25, depth=150_000)
+    _, _, rec = jobs.run_oracle(job)
+    obs = rec.obs_text()
+    marked = jobs.native_replay(obs, by_poll=True)
+    counts = check_orion_invariants(obs, marked, 150_000)
+    assert all(v > 0 for v in counts.values()), counts
+    lines = marked.splitlines()
+    # move the first high-priority dispatch one poll later
+    i = next(k for k, l in enumerate(lines) if l.startswith("D 2 "))
+    j = next(k for k in range(i + 1, len(lines)) if lines[k] == "P")
+    moved = lines[:i] + lines[i + 1:j + 1] + [lines[i]] + lines[j + 1:]
+    try:
+        check_orion_invariants(obs, "\n".join(moved) + "\n", 150_000)
+    except AssertionError:
+        return
+    raise AssertionError("a displaced high-priority dispatch went unnoticed")
