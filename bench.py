@@ -5,9 +5,12 @@ MI355X, with the hand-written kernels' roofline and a CPU baseline beside it.
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One "step" is one high-priority request through the whole hot path
-(interception -> queue -> policy -> dispatch).  K requests are measured after
-the client protocol's own 10 warm-up requests; W is the number of untimed
-launches before the kernel-level timings.  Prints ONE JSON line.
+(interception -> queue -> policy -> dispatch).  K requests are measured
+isolated and K co-located, in --repeats alternating runs of K / repeats
+requests, each after the client protocol's own 10 untimed warm-up requests
+(fixed by the protocol; W does not change it).  W is the number of untimed
+launches before the triad timings; the GEMM always gets 100, which is what the
+power-limited package needs to settle.  Prints ONE JSON line.
 
 Work done, in order (child processes first, so that this process has not touched
 the GPU when it starts them):
@@ -241,7 +244,7 @@ def main():
     import torch
     from orion_amd import kernel_pair as kp
     reps = max(20, min(200, args.steps // 6))
-    alone = kp.measure_alone(reps=reps)
+    alone = kp.measure_alone(reps=reps, warmup=max(1, args.warmup))
     pairs = [kp.measure_pair(m, reps=reps) for m in (32, 64, 128, 0)]
     gemm = alone["gemm"]
     flops = 2 * kp.GEMM_N ** 3

@@ -60,7 +60,7 @@ def _time_launches(stream, launch, reps, warmup=2):
 
 
 def measure_alone(gemm_n=GEMM_N, triad_elems=TRIAD_ELEMS, masks=(32, 64, 128, 0),
-                  reps=10, device="cuda:0"):
+                  reps=10, device="cuda:0", warmup=2):
     """Each kernel alone: GEMM on the whole GPU, triad per CU-mask size."""
     a, b = _inputs_gemm(gemm_n, device)
     c = torch.empty(gemm_n, gemm_n, device=device, dtype=torch.bfloat16)
@@ -81,7 +81,8 @@ def measure_alone(gemm_n=GEMM_N, triad_elems=TRIAD_ELEMS, masks=(32, 64, 128, 0)
     out["triad"] = {}
     for m in masks:
         s = kernels.cu_masked_stream(m)
-        ms = _time_launches(s, lambda st: kernels.triad(ta, tb, tc, 1.7, stream=st), reps)
+        ms = _time_launches(s, lambda st: kernels.triad(ta, tb, tc, 1.7, stream=st), reps,
+                            warmup=warmup)
         gbs = 12 * triad_elems / ms / 1e6
         out["triad"][str(m or 256)] = {"ms": ms, "gbs": gbs, "frac_of_peak": gbs / HBM_PEAK_GBS}
     return out
