@@ -2,7 +2,7 @@
 // (rocprofv3 --kernel-trace / --pmc -- orion_amd/bench_kernels): it uses the
 // system HIP runtime only, so a profiler sees exactly these kernels.
 //
-//   bench_kernels [--reps N] [--warmup N] [--gemm-n N] [--triad-elems N] [--mask CUS]
+//   bench_kernels [--reps N] [--warmup N] [--gemm-n N] [--triad-elems N] [--triad-skew BYTES] [--mask CUS]
 //                 [--pair 1]
 //
 // --pair 1 runs the two kernels at the same time instead: the GEMM on a stream
@@ -127,13 +127,14 @@ static void run_pair(hipStream_t sg, hipStream_t st, GemmCtx* g, TriadCtx* t, in
 
 int main(int argc, char** argv) {
   int reps = 200, warmup = 100, gemm_n = 8192, mask = 0, pair = 0;
-  size_t elems = (size_t)1 << 28;
+  size_t elems = (size_t)1 << 28, skew = 0;
   for (int i = 1; i + 1 < argc; i += 2) {
     if (!strcmp(argv[i], "--reps")) reps = atoi(argv[i + 1]);
     else if (!strcmp(argv[i], "--warmup")) warmup = atoi(argv[i + 1]);
     else if (!strcmp(argv[i], "--gemm-n")) gemm_n = atoi(argv[i + 1]);
     else if (!strcmp(argv[i], "--triad-elems")) elems = strtoull(argv[i + 1], nullptr, 10);
     else if (!strcmp(argv[i], "--mask")) mask = atoi(argv[i + 1]);
+    else if (!strcmp(argv[i], "--triad-skew")) skew = strtoull(argv[i + 1], nullptr, 10);
     else if (!strcmp(argv[i], "--pair")) pair = atoi(argv[i + 1]);
   }
   hipStream_t full = nullptr, masked = nullptr;
@@ -150,9 +151,15 @@ int main(int argc, char** argv) {
   hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)g.B, mat / 2, 2u, 1);
   TriadCtx t;
   t.n = elems;
-  CHECK(hipMalloc((void**)&t.a, elems * 4));
+  // --triad-skew S (a multiple of 16): c starts S bytes and a 2 S bytes further
+  // into their allocations than b, so the three streams do not walk the memory
+  // channels in lockstep
+  if (skew % 16) return 4;
+  CHECK(hipMalloc((void**)&t.a, elems * 4 + 2 * skew));
   CHECK(hipMalloc((void**)&t.b, elems * 4));
-  CHECK(hipMalloc((void**)&t.c, elems * 4));
+  CHECK(hipMalloc((void**)&t.c, elems * 4 + skew));
+  t.a = (float*)((char*)t.a + 2 * skew);
+  t.c = (float*)((char*)t.c + skew);
   hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)t.b, elems, 3u, 0);
   hipLaunchKernelGGL(init_uniform, dim3(4096), dim3(256), 0, full, (uint32_t*)t.c, elems, 4u, 0);
   CHECK(hipStreamSynchronize(full));
