@@ -39,6 +39,9 @@ def _check_replay(record_dir):
     if seg[3] == "orion" and not hp_trains:
         from tests.test_policy_properties import check_orion_invariants
         check_orion_invariants(obs, jobs.native_replay(obs, by_poll=True), int(seg[4]))
+    elif seg[3] == "reef":
+        from tests.test_policy_properties import check_reef_rule
+        check_reef_rule(obs, jobs.native_replay(obs, by_poll=True))
     return dec
 
 

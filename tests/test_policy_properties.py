@@ -25,6 +25,10 @@ bookkeeping (seen[], iteration counts, the running best-effort duration sum):
 
 Profile durations are whole numbers below 2^24, so the reference's float/long
 sum is exact here.
+
+REEF (schedule_reef, :93-165) is simpler: which clients a poll dispatches is a
+function of what the poll saw and three counters, so the whole rule is checked,
+not only invariants of it.
 """
 
 import csv
@@ -154,6 +158,114 @@ def check_orion_invariants(obs_text, dec_text, depth):
                     seen[c], iters[c], event_ids[c] = 0, iters[c] + 1, 0
     assert at == len(dec)
     return checked
+
+
+def check_reef_rule(obs_text, dec_text):
+    """The REEF rule, poll by poll (reference: schedule_reef,
+    scheduler_eval.cpp:93-165): which clients a poll dispatches is a function of
+    the heads it saw, the iteration counts, the profile rows at seen[] and the
+    penalty counter."""
+    obs, dec = obs_text.splitlines(), dec_text.splitlines()
+    at = 0
+    n = None
+    nk, max_iters, prof, seen, iters = {}, {}, {}, {}, {}
+    penalty = 0                               # a member of the scheduler: never reset
+    kinds = {"first": 0, "paired": 0, "unpaired": 0, "released": 0, "held": 0}
+    for line in obs:
+        p = line.split(" ")
+        if p[0] == "J":
+            n = int(p[1])
+            hp = n - 1
+        elif p[0] == "K":
+            c = int(p[1])
+            nk[c], max_iters[c], prof[c] = int(p[2]), int(p[3]), rows_of(p[5])
+            seen[c], iters[c] = 0, 0
+        elif p[0] == "X":
+            c = int(p[1])
+            nk[c], prof[c] = int(p[2]), rows_of(p[3])
+            assert dec[at] == f"X {c}"
+            at += 1
+        elif p[0] == "S":
+            assert dec[at] == "S" and p[3] == "reef"
+            at += 1
+            depth = int(p[4])
+        elif p[0] == "E":
+            assert dec[at] == "E"
+            at += 1
+        elif p[0] == "P":
+            assert dec[at] == "P"
+            at += 1
+            heads = p[2]
+            block = []
+            while at < len(dec) and dec[at][0] in "DFT":
+                block.append(dec[at].split(" "))
+                at += 1
+            got = [int(b[1]) for b in block if b[0] == "D"]
+            present = [c for c in range(n) if heads[c] in RECORD]
+            for c in range(n):
+                if seen[c] == nk[c]:
+                    assert heads[c] == "-"
+            if n == 1:
+                want = present
+            else:
+                first = [c for c in present
+                         if heads[c] == "m" or iters[c] <= 10 or iters[hp] >= max_iters[hp]]
+                if first:                                         # :108-116
+                    want = first[:1]
+                    kinds["first"] += 1
+                elif hp in present:                               # :119-141
+                    hp_row = prof[hp][seen[hp]]
+                    fits = [c for c in present if c != hp
+                            and prof[c][seen[c]][2] <= hp_row[2]
+                            and prof[c][seen[c]][1] >= hp_row[1]]
+                    want = [hp] + fits[:1]
+                    kinds["paired" if fits else "unpaired"] += 1
+                else:                                             # :143-163
+                    penalty += len(present)
+                    if penalty >= depth:
+                        want, penalty = present, 0
+                        kinds["released"] += bool(present)
+                    else:
+                        want = []
+                        kinds["held"] += bool(present)
+            assert got == want, (line, block, want)
+            for b in block:
+                c = int(b[1])
+                if b[0] == "D" and b[3] == "k":
+                    seen[c] += 1
+                elif b[0] == "F":
+                    assert seen[c] == nk[c]
+                    seen[c], iters[c] = 0, iters[c] + 1
+    assert at == len(dec)
+    return kinds
+
+
+@settings(max_examples=100, deadline=None,
+          suppress_health_check=[HealthCheck.function_scoped_fixture, HealthCheck.too_slow])
+@given(seed=st.integers(0, 10_000), n_clients=st.integers(1, 5), hp_iters=st.integers(11, 30))
+def test_reef_rule_on_the_native_core(tmp_path_factory, seed, n_clients, hp_iters):
+    tmp = str(tmp_path_factory.mktemp("job"))
+    job = jobs.make_job(tmp, seed, n_clients=n_clients, algo=po.ALGO_REEF, hp_train=False,
+                        hp_iters=hp_iters)
+    _, _, rec = jobs.run_oracle(job)
+    obs = rec.obs_text()
+    marked = jobs.native_replay(obs, by_poll=True)
+    assert "".join(l + "\n" for l in marked.splitlines() if l != "P") == rec.dec.text()
+    check_reef_rule(obs, marked)
+
+
+def test_reef_rule_fires_every_branch(tmp_path):
+    seen = {}
+    for seed in range(6):
+        job = jobs.make_job(str(tmp_path), seed, n_clients=3, algo=po.ALGO_REEF, hp_iters=25)
+        _, _, rec = jobs.run_oracle(job)
+        for k, v in check_reef_rule(rec.obs_text(),
+                                    jobs.native_replay(rec.obs_text(), by_poll=True)).items():
+            seen[k] = seen.get(k, 0) + v
+    assert all(v > 0 for v in seen.values()), seen
+    d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fake_reef_2be")
+    obs = open(os.path.join(d, "observations.log")).read().replace("@DIR@", d)
+    check_reef_rule(obs, jobs.native_replay(obs, by_poll=True))
 
 
 @settings(max_examples=150, deadline=None,
