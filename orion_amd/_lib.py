@@ -35,3 +35,16 @@ def load(path, mode=ctypes.DEFAULT_MODE):
     lib = ctypes.CDLL(path, mode=mode)
     _cache[path] = lib
     return lib
+
+
+def loaded(path):
+    """The handle ``load`` returned for ``path``, or None."""
+    return _cache.get(path)
+
+
+def unload(path):
+    """Closes a library loaded here; its handle must not be used afterwards."""
+    lib = _cache.pop(path, None)
+    if lib is not None:
+        import _ctypes
+        _ctypes.dlclose(lib._handle)

@@ -4,6 +4,7 @@ torch is used only as the owner of device memory and streams; the arithmetic
 runs in the HIP kernels behind the C ABI declared in ``include/orion_kernels.h``.
 """
 
+import atexit
 import ctypes
 
 import torch
@@ -39,6 +40,9 @@ def lib():
     return handle
 
 
+_streams = []          # raw handles of the streams made here, destroyed at exit
+
+
 def cu_masked_stream(cu_count, device=0):
     """A ``torch.cuda.ExternalStream`` over a stream limited to ``cu_count``
     compute units (the whole GPU for ``cu_count <= 0``)."""
@@ -46,7 +50,25 @@ def cu_masked_stream(cu_count, device=0):
     rc = lib().orion_stream_create(int(cu_count), ctypes.byref(out))
     if rc != 0:
         raise KernelError("orion_stream_create", rc)
+    _streams.append(out.value)
     return torch.cuda.ExternalStream(out.value, device=device)
+
+
+@atexit.register
+def _shutdown():
+    """Gives back what this module took from the HIP runtime while the runtime
+    is still up: waits for the device, destroys the streams made here and
+    unloads the kernel library (which un-registers its code object).  Left to
+    process exit, the library's own finaliser runs after the interpreter and
+    whatever else hooks the runtime (a profiler) have shut down."""
+    handle = _lib.loaded(_lib.KERNELS_LIB)
+    if handle is None:
+        return
+    if torch.cuda.is_initialized():
+        torch.cuda.synchronize()
+    while _streams:
+        handle.orion_stream_destroy(ctypes.c_void_p(_streams.pop()))
+    _lib.unload(_lib.KERNELS_LIB)
 
 
 def _stream_ptr(stream):
