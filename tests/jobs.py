@@ -159,15 +159,8 @@ def policy_lib():
 
 def native_replay(obs_text, sequential_fix=True, by_poll=False):
     """Decision log of the native policy core for an observation log."""
-    lib = policy_lib()
-    out, err = ctypes.c_void_p(), ctypes.c_void_p()
-    fn = lib.orion_policy_replay_by_poll if by_poll else lib.orion_policy_replay
-    rc = fn(obs_text.encode(), int(sequential_fix), ctypes.byref(out), ctypes.byref(err))
+    from orion_amd import replay
     try:
-        if rc != 0:
-            msg = ctypes.string_at(err).decode() if err else f"rc={rc}"
-            raise RuntimeError(f"native replay failed: {msg}")
-        return ctypes.string_at(out).decode()
-    finally:
-        lib.orion_policy_free(out)
-        lib.orion_policy_free(err)
+        return replay.native_replay(obs_text, by_poll=by_poll, sequential_fix=sequential_fix)
+    except replay.ReplayError as e:
+        raise RuntimeError(f"native replay failed: {e}") from e
