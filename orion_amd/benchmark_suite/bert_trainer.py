@@ -126,5 +126,5 @@ def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
         result = cc.run_client(tid, train, num_iters, sleep_times, barriers, step,
                                backend, drop=50 if not train and num_iters > 60 else 10,
                                extra=extra)
-    print(f"Client {tid} finished: {result}", flush=True)
+    print(f"Client {tid} finished: {cc.brief(result)}", flush=True)
     return result

@@ -73,6 +73,11 @@ def latency_summary(timings, batch_idx, total_time, train, drop=WARMUP_ITERS):
     return {"throughput": throughput}
 
 
+def brief(data):
+    """A result without its per-request list, for the one-line report."""
+    return {k: v for k, v in data.items() if k != "latencies_ms"}
+
+
 def write_result(tid, data):
     out_dir = os.environ.get("ORION_RESULT_DIR", ".")
     os.makedirs(out_dir, exist_ok=True)
@@ -199,6 +204,6 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
     if not train:
         # every measured request, in arrival order (the reference's file holds
         # the percentiles only): lets runs be pooled
-        data["latencies_ms"] = [round(t * 1000, 4) for t in timings[drop:]]
+        data["latencies_ms"] = [round(float(t) * 1000, 4) for t in timings[drop:]]
     write_result(tid, data)
     return data

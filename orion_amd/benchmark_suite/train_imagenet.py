@@ -131,5 +131,5 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                 torch.cuda.synchronize()
         result = cc.run_client(tid, train, num_iters, sleep_times, barriers, step,
                                backend, extra=extra)
-    print(f"Client {tid} finished: {result}", flush=True)
+    print(f"Client {tid} finished: {cc.brief(result)}", flush=True)
     return result

@@ -106,5 +106,5 @@ def transformer_loop(batchsize, train, num_iters, rps, uniform, dummy_data, loca
                 step(-1 - i)
         result = cc.run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
                                extra=extra)
-    print(f"Client {tid} finished: {result}", flush=True)
+    print(f"Client {tid} finished: {cc.brief(result)}", flush=True)
     return result
