@@ -84,13 +84,13 @@ def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_gr
 
 def policy_replay(record_dir):
     """Bit-exact check and replay rate over the co-located run's own log."""
-    from oracle import obslog
-    from tests import jobs
+    from oracle import obslog          # the checker (CPU baseline of the policy)
+    from orion_amd import replay
     obs = open(os.path.join(record_dir, "observations.log")).read()
     dec = open(os.path.join(record_dir, "decisions.log")).read()
     n_dec = dec.count("\nD ") + dec.startswith("D ")
     t0 = time.perf_counter()
-    native = jobs.native_replay(obs)
+    native = replay.native_replay(obs)
     t_native = time.perf_counter() - t0
     # the oracle is pure Python: replay a bounded prefix (whole segments)
     lines = obs.splitlines(keepends=True)
