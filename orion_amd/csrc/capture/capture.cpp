@@ -18,6 +18,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <sys/syscall.h>
+#include <time.h>
 #include <unistd.h>
 
 using namespace orion;
@@ -260,6 +261,7 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
     abort();
   }
   g_state.armed.store(0, std::memory_order_release);
+  g_state.scheduler_polling.store(0, std::memory_order_release);
   pinning_undo();
   pinning_reset(num_clients + 1);
   g_state.num_clients = num_clients;
@@ -368,6 +370,14 @@ int stop(void) {
 
 namespace {
 
+double stuck_limit_s() {
+  static const double limit = [] {
+    const char* e = getenv("ORION_STUCK_LIMIT_S");
+    return e && atof(e) > 0 ? atof(e) : 20.0;
+  }();
+  return limit;
+}
+
 // Pushes `r` to client idx's queue and waits until the scheduler has taken it
 // (or, for free(), only until it is queued: intercept_temp.cpp:214-236).
 // Returns the HIP status of the call.
@@ -410,7 +420,32 @@ int submit(int idx, Record& r, bool wait) {
   if (!wait) return (int)hipSuccess;
 
   spins = 0;
+  unsigned long waited = 0;
+  double idle_since = 0.0;
   while (ch.head.load(std::memory_order_acquire) <= ticket) {
+    // Clients submit only while the scheduler polls; between two calls of
+    // schedule() they wait at a rendezvous.  A record that sits here for long
+    // with the scheduler outside its loop can never be taken (the usual cause:
+    // the iteration holds more kernel records than the client's profile names,
+    // so the scheduler counted it complete and left): say so instead of
+    // spinning forever, as the reference would (intercept_temp.cpp:404-416).
+    if ((++waited & 0xfffff) == 0) {
+      if (g_state.scheduler_polling.load(std::memory_order_acquire)) {
+        idle_since = 0.0;
+      } else {
+        timespec ts;
+        clock_gettime(CLOCK_MONOTONIC, &ts);
+        const double now = (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+        if (idle_since == 0.0) idle_since = now;
+        if (now - idle_since > stuck_limit_s()) {
+          fprintf(stderr,
+                  "orion: client %d has had a record (type %d) queued for %.0f s while the "
+                  "scheduler is not polling; its iteration probably holds more kernel records "
+                  "than its profile's num_kernels\n", idx, r.type, now - idle_since);
+          abort();
+        }
+      }
+    }
     if (!g_state.armed.load(std::memory_order_acquire)) {
       // The scheduler has left its loop for good.  Whatever it did not take is
       // run here, in order, on the stream the call named.

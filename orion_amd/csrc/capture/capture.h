@@ -157,6 +157,7 @@ struct alignas(64) ClientChannel {
 struct CaptureState {
   std::atomic<int> armed;        // 0 = pass everything through
   std::atomic<uint32_t> epoch;   // bumped by every arm(): invalidates thread caches
+  std::atomic<int> scheduler_polling;  // 1 while the scheduler thread is inside schedule()
   int num_clients;
   pid_t client_tids[kMaxClients];
   pid_t scheduler_tid;

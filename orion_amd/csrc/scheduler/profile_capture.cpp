@@ -208,6 +208,7 @@ int orion_profile_run(int until_iteration) {
   CaptureRun& run = g_run;
   const HipApi* hip = run.hip;
   ClientChannel& ch = orion_capture_state()->channels[0];
+  orion_capture_state()->scheduler_polling.store(1, std::memory_order_release);
   while (run.iteration < until_iteration) {
     const uint64_t head = ch.head.load(std::memory_order_relaxed);
     if (ch.tail.load(std::memory_order_acquire) == head) {
@@ -241,6 +242,7 @@ int orion_profile_run(int until_iteration) {
     }
     ch.head.store(head + 1, std::memory_order_release);
   }
+  orion_capture_state()->scheduler_polling.store(0, std::memory_order_release);
   return 0;
 }
 

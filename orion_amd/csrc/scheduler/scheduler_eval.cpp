@@ -185,6 +185,15 @@ class LiveHost : public PolicyHost {
     return true;
   }
 
+  // Class of the record waiting at the head of a client's queue (REC_NONE if
+  // none), without the bookkeeping peek() does.
+  int waiting_class(int client) const {
+    ClientChannel& ch = cap_->channels[client];
+    const uint64_t head = ch.head.load(std::memory_order_relaxed);
+    if (ch.tail.load(std::memory_order_acquire) == head) return REC_NONE;
+    return rec_class_of(ch.slots[head & (kQueueSlots - 1)].type);
+  }
+
   int64_t iteration_us(int client) override {
     return std::chrono::duration_cast<std::chrono::microseconds>(
                Clock::now() - iter_start_[(size_t)client]).count();
@@ -194,6 +203,22 @@ class LiveHost : public PolicyHost {
     ClientChannel& ch = cap_->channels[d.client];
     const uint64_t head = ch.head.load(std::memory_order_relaxed);
     Record* rec = &ch.slots[head & (kQueueSlots - 1)];
+
+    // A client ends every iteration with block(): when the policy starts
+    // counting a new iteration for it (profile row 0) it must have called
+    // block() for all the iterations already released.  If it has not, its
+    // iteration holds more kernel records than its profile's num_kernels and
+    // every later kernel would be matched with the wrong profile row (the
+    // reference runs on silently, scheduler_eval.cpp:281-282, :409-420).
+    if (d.rec_class == REC_KERNEL && d.op_index == 0 && policy_) {
+      const long long done = policy_->cur_iters()[(size_t)d.client];
+      const long long blocked = ch.block_calls.load(std::memory_order_acquire);
+      if (blocked < done)
+        die("client " + std::to_string(d.client) + " submits more kernel records per "
+            "iteration than the " + std::to_string(policy_->num_kernels()[(size_t)d.client]) +
+            " its profile names: " + std::to_string(done) + " iterations completed by count, "
+            "block() called " + std::to_string(blocked) + " times");
+    }
 
     // Stream: the owner's stream set, at the slot the policy placed the kernel
     // in; records that are not kernels stay where the client's work is.
@@ -502,8 +527,22 @@ void* schedule(void* /*scheduler*/, int num_clients, bool profile_mode, int /*it
     g.recorder->begin_schedule(a);
     host = g.recorder.get();
   }
+  orion_capture_state()->scheduler_polling.store(1, std::memory_order_release);
   g.policy->schedule(*host, a);
+  orion_capture_state()->scheduler_polling.store(0, std::memory_order_release);
   g.host->set_direct(hp, false);
+  if (warmup) {
+    // A warm-up phase ends with every client between two iterations, on its way
+    // to the rendezvous with this thread.  A kernel still waiting in a queue
+    // belongs to an iteration the policy has already counted as complete: the
+    // client's iteration holds more kernel records than its profile names, and
+    // it would wait for this thread forever while this thread waits for it.
+    for (int i = 0; i < g.n; ++i)
+      if (g.host->waiting_class(i) == REC_KERNEL)
+        die("client " + std::to_string(i) + " submits more kernel records per iteration "
+            "than the " + std::to_string(g.policy->num_kernels()[(size_t)i]) +
+            " its profile names: one is still queued after the iteration was released");
+  }
   if (g.recorder) {
     g.recorder->end_schedule();
     flush_recording();

@@ -57,8 +57,9 @@ records_per_iter = list(kernels_per_iter)                 # what the scheduler c
 if hp_graph:
     records_per_iter[-1] = 1
 if os.environ.get("FAKE_RUNNER_MISCOUNT"):
-    # tell the scheduler one kernel more than client 0 submits per iteration
-    records_per_iter[0] += 1
+    # tell the scheduler one kernel more (or, with -1, one fewer) than client 0
+    # submits per iteration
+    records_per_iter[0] += int(os.environ["FAKE_RUNNER_MISCOUNT"])
 iters = [10_000] * n_be + [hp_iters]
 
 

@@ -140,3 +140,23 @@ def test_kernel_count_mismatch_ends_the_job_with_a_report(tmp_path):
     # client 0 has handed over all 5 of the 6 kernels the scheduler was told about
     assert "client 0: 5 of 6 kernel records seen this iteration" in proc.stderr
     assert "block() calls 1, iterations released 0" in proc.stderr
+
+
+def test_more_kernels_than_the_profile_names_is_reported_at_once(tmp_path):
+    """The other direction of the mismatch: a client whose iteration holds more
+    kernel records than its profile.  The reference matches every later kernel
+    with the wrong profile row and runs on; here the scheduler sees the first
+    kernel of the "next" iteration arrive before the client has called block()
+    and ends the job."""
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), str(tmp_path),
+         "orion", "1", "20"],
+        capture_output=True, text=True, timeout=120,
+        env=dict(os.environ, FAKE_RUNNER_MISCOUNT="-1", ORION_STUCK_LIMIT_S="2"))
+    assert proc.returncode != 0
+    # seen by the scheduler (the extra kernel arrives while it polls, or is still
+    # queued when a warm-up phase ends) or, when the scheduler has already left
+    # for the rendezvous, by the client that waits for it in vain
+    assert ("client 0 submits more kernel records per iteration than the 4 its profile names"
+            in proc.stderr
+            or "client 0 has had a record (type" in proc.stderr), proc.stderr[-2000:]
