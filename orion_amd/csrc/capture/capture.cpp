@@ -124,6 +124,9 @@ hipStream_t named_stream(const Record& r) {
   if (r.type <= RT_MODULE_COOP_LAUNCH) return r.u.module.stream;
   if (r.type <= RT_MEMCPY_2D_ASYNC) return r.u.copy.stream;
   if (r.type == RT_GRAPH_LAUNCH) return r.u.graph.stream;
+  if (r.type == RT_MEMCPY_2D) return nullptr;
+  if (r.type == RT_MALLOC_ASYNC) return r.u.malloc_.stream;
+  if (r.type == RT_FREE_ASYNC) return r.u.free_.stream;
   if (r.type >= RT_MEMSET) return r.u.set.stream;
   return nullptr;
 }
@@ -152,6 +155,18 @@ int execute_on_caller(Record& r, hipStream_t stream) {
       err = hip->hipMemsetAsync(r.u.set.dst, r.u.set.value, r.u.set.count, stream);
       if (err == hipSuccess) err = hip->hipStreamSynchronize(stream);
       break;
+    case RT_MEMCPY_2D:
+      err = hip->hipMemcpy2DAsync(r.u.copy.dst, r.u.copy.dpitch, r.u.copy.src, r.u.copy.spitch,
+                                  r.u.copy.width, r.u.copy.height, r.u.copy.kind, stream);
+      if (err == hipSuccess) err = hip->hipStreamSynchronize(stream);
+      break;
+    case RT_MALLOC_ASYNC:   // ordered after the client's earlier work, where it now runs
+      err = hip->hipMallocAsync ? hip->hipMallocAsync(r.u.malloc_.ptr, r.u.malloc_.size, stream)
+                                : hipErrorNotSupported;
+      break;
+    case RT_FREE_ASYNC:
+      err = hip->hipFreeAsync ? hip->hipFreeAsync(r.u.free_.ptr, stream) : hipErrorNotSupported;
+      break;
     default:
       err = hipErrorInvalidValue;
   }
@@ -171,7 +186,8 @@ enum { ORION_GRANTED_TO_CALLER = orion::kRecordGranted };
 
 bool orion_record_runs_on_caller(int type) {
   return type == RT_MALLOC || type == RT_FREE || type == RT_MEMCPY ||
-         type == RT_MEMCPY_WITH_STREAM || type == RT_MEMSET;
+         type == RT_MEMCPY_WITH_STREAM || type == RT_MEMSET || type == RT_MEMCPY_2D ||
+         type == RT_MALLOC_ASYNC || type == RT_FREE_ASYNC;
 }
 
 // Issues a record's HIP call on `stream` (scheduler thread).  Returns the HIP
@@ -590,7 +606,31 @@ hipError_t hipMalloc(void** ptr, size_t size) {
   if (idx < 0) return orion_hip_api()->hipMalloc(ptr, size);
   Record r;
   r.type = RT_MALLOC;
-  r.u.malloc_ = {ptr, size};
+  r.u.malloc_ = {ptr, size, nullptr};
+  return (hipError_t)submit(idx, r, true);
+}
+
+// Stream-ordered allocation (an optional allocator backend of PyTorch, rocBLAS
+// workspaces): ordered on the stream the client's work has been moved to.
+hipError_t hipMallocAsync(void** ptr, size_t size, hipStream_t stream) {
+  const int idx = client_for_call(stream);
+  if (idx < 0 || !orion_hip_api()->hipMallocAsync)
+    return orion_hip_api()->hipMallocAsync ? orion_hip_api()->hipMallocAsync(ptr, size, stream)
+                                           : hipErrorNotSupported;
+  Record r;
+  r.type = RT_MALLOC_ASYNC;
+  r.u.malloc_ = {ptr, size, stream};
+  return (hipError_t)submit(idx, r, true);
+}
+
+hipError_t hipFreeAsync(void* ptr, hipStream_t stream) {
+  const int idx = client_for_call(stream);
+  if (idx < 0 || !orion_hip_api()->hipFreeAsync)
+    return orion_hip_api()->hipFreeAsync ? orion_hip_api()->hipFreeAsync(ptr, stream)
+                                         : hipErrorNotSupported;
+  Record r;
+  r.type = RT_FREE_ASYNC;
+  r.u.free_ = {ptr, stream};
   return (hipError_t)submit(idx, r, true);
 }
 
@@ -599,7 +639,7 @@ hipError_t hipFree(void* ptr) {
   if (idx < 0) return orion_hip_api()->hipFree(ptr);
   Record r;
   r.type = RT_FREE;
-  r.u.free_ = {ptr};
+  r.u.free_ = {ptr, nullptr};
   return (hipError_t)submit(idx, r, true);
 }
 
@@ -642,6 +682,17 @@ hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t sp
   Record r;
   r.type = RT_MEMCPY_2D_ASYNC;
   r.u.copy = {dst, src, 0, kind, stream, dpitch, spitch, width, height};
+  return (hipError_t)submit(idx, r, true);
+}
+
+hipError_t hipMemcpy2D(void* dst, size_t dpitch, const void* src, size_t spitch,
+                       size_t width, size_t height, hipMemcpyKind kind) {
+  const int idx = client_for_call(nullptr);
+  if (idx < 0)
+    return orion_hip_api()->hipMemcpy2D(dst, dpitch, src, spitch, width, height, kind);
+  Record r;
+  r.type = RT_MEMCPY_2D;
+  r.u.copy = {dst, src, 0, kind, nullptr, dpitch, spitch, width, height};
   return (hipError_t)submit(idx, r, true);
 }
 

@@ -46,6 +46,9 @@ enum RecType : int32_t {
   RT_MEMSET_D16_ASYNC,         // hipMemsetD16Async
   RT_MEMSET_D8_ASYNC,          // hipMemsetD8Async
   RT_GRAPH_LAUNCH,             // hipGraphLaunch: a whole captured graph, one record
+  RT_MEMCPY_2D,                // hipMemcpy2D (blocking)
+  RT_MALLOC_ASYNC,             // hipMallocAsync
+  RT_FREE_ASYNC,               // hipFreeAsync
   RT_COUNT
 };
 
@@ -53,9 +56,9 @@ enum RecType : int32_t {
 // `seen`, src/scheduler/utils_sched.cpp:242-513).
 inline int rec_class_of(int type) {
   if (type <= RT_MODULE_COOP_LAUNCH || type == RT_GRAPH_LAUNCH) return REC_KERNEL;
-  if (type <= RT_MEMCPY_2D_ASYNC) return REC_MEMCPY;
-  if (type == RT_MALLOC) return REC_MALLOC;
-  if (type == RT_FREE) return REC_FREE;
+  if (type <= RT_MEMCPY_2D_ASYNC || type == RT_MEMCPY_2D) return REC_MEMCPY;
+  if (type == RT_MALLOC || type == RT_MALLOC_ASYNC) return REC_MALLOC;
+  if (type == RT_FREE || type == RT_FREE_ASYNC) return REC_FREE;
   return REC_MEMSET;
 }
 
@@ -104,9 +107,11 @@ struct Record {
     struct {
       void** ptr;
       size_t size;
+      hipStream_t stream;  // hipMallocAsync only
     } malloc_;
     struct {
       void* ptr;
+      hipStream_t stream;  // hipFreeAsync only
     } free_;
     struct {
       void* dst;

@@ -57,6 +57,10 @@ namespace orion {
      hipStream_t, void**))                                                                  \
   X(hipMalloc, hipError_t, (void**, size_t))                                                \
   X(hipFree, hipError_t, (void*))                                                           \
+  X(hipMallocAsync, hipError_t, (void**, size_t, hipStream_t))                              \
+  X(hipFreeAsync, hipError_t, (void*, hipStream_t))                                         \
+  X(hipMemcpy2D, hipError_t,                                                                \
+    (void*, size_t, const void*, size_t, size_t, size_t, hipMemcpyKind))                    \
   X(hipMemcpy, hipError_t, (void*, const void*, size_t, hipMemcpyKind))                     \
   X(hipMemcpyAsync, hipError_t, (void*, const void*, size_t, hipMemcpyKind, hipStream_t))   \
   X(hipMemcpyWithStream, hipError_t,                                                        \

@@ -43,6 +43,10 @@ cap.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
 cap.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 
 cap.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+cap.hipMallocAsync.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t, ctypes.c_void_p]
+cap.hipFreeAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+cap.hipMemcpy2D.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                            ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
 
 
 class FakeGraphExec(ctypes.Structure):      # mirrors tests/fakehip/fakehip.cpp
@@ -103,6 +107,15 @@ def client(tid):
     assert cap.hipMalloc(ctypes.byref(dev_x), N * 4) == 0
     zeros = np.zeros(N, dtype=np.float32)
     cap.hipMemcpy(dev_y, zeros.ctypes.data, N * 4, 1)
+    # stream-ordered allocation and a blocking 2-D copy: granted back to this
+    # thread, on the stream the scheduler assigned
+    scratch = ctypes.c_void_p()
+    assert cap.hipMallocAsync(ctypes.byref(scratch), 2 * N * 4, None) == 0
+    assert cap.hipMemcpy2D(scratch, N * 4, host_x.ctypes.data, N * 4, N * 4, 1, 1) == 0
+    back = np.empty(N, dtype=np.float32)
+    assert cap.hipMemcpy2D(back.ctypes.data, N * 4, scratch, N * 4, N * 4, 1, 2) == 0
+    assert np.array_equal(back, host_x)
+    assert cap.hipFreeAsync(scratch, None) == 0
     it = 0
     n_c, a_c = ctypes.c_int(N), ctypes.c_float(0.5)
     c_c = ctypes.c_float(0.125)
@@ -198,6 +211,8 @@ for c in range(n_clients):
 
 print(json.dumps({
     "alive": alive, "iters_done": iters_done, "outputs_equal": ok_outputs,
+    "async_allocs": [[s, t] for k, s, t in log if k == 3 and s != 0],
+    "async_frees": [[s, t] for k, s, t in log if k == 4 and s != 0],
     "placement": placement[:n_clients], "scheduler_placement": placement[n_clients],
     "scheduler_mask_after": sched_after, "allowed_cpus": sorted(os.sched_getaffinity(0)),
     "launch_tids": launch_tids, "sched_tid": sched_tid, "client_tids": tids,

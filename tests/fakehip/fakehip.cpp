@@ -194,6 +194,16 @@ hipError_t hipFree(void* p) {
   free(p);
   return hipSuccess;
 }
+hipError_t hipMallocAsync(void** p, size_t n, hipStream_t s) {
+  *p = malloc(n ? n : 1);
+  log_call(3, s, (uint64_t)*p, n);
+  return *p ? hipSuccess : hipErrorOutOfMemory;
+}
+hipError_t hipFreeAsync(void* p, hipStream_t s) {
+  log_call(4, s, (uint64_t)p, 0);
+  free(p);
+  return hipSuccess;
+}
 hipError_t hipMemcpyAsync(void* d, const void* s_, size_t n, hipMemcpyKind, hipStream_t s) {
   log_call(1, s, (uint64_t)d, n);
   memcpy(d, s_, n);
@@ -212,6 +222,10 @@ hipError_t hipMemcpy2DAsync(void* d, size_t dp, const void* s_, size_t sp, size_
   for (size_t r = 0; r < h; ++r) memcpy((char*)d + r * dp, (const char*)s_ + r * sp, w);
   occupy(s, g_copy_ns);
   return hipSuccess;
+}
+hipError_t hipMemcpy2D(void* d, size_t dp, const void* s_, size_t sp, size_t w, size_t h,
+                       hipMemcpyKind k) {
+  return hipMemcpy2DAsync(d, dp, s_, sp, w, h, k, nullptr);
 }
 hipError_t hipMemsetAsync(void* d, int v, size_t n, hipStream_t s) {
   log_call(2, s, (uint64_t)d, n);

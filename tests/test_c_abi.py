@@ -59,7 +59,8 @@ def test_interposed_hip_symbols_are_exported():
               "hipExtModuleLaunchKernel", "hipHccModuleLaunchKernel",
               "hipModuleLaunchCooperativeKernel", "hipLaunchCooperativeKernel",
               "hipGraphLaunch",
-              "hipMalloc", "hipFree", "hipMemcpy", "hipMemcpyAsync",
+              "hipMalloc", "hipFree", "hipMallocAsync", "hipFreeAsync", "hipMemcpy2D",
+              "hipMemcpy", "hipMemcpyAsync",
               "hipMemcpyWithStream", "hipMemcpy2DAsync", "hipMemset",
               "hipMemsetAsync", "hipMemsetD32Async", "hipMemsetD16Async",
               "hipMemsetD8Async", "hipStreamSynchronize", "hipStreamQuery",

@@ -71,6 +71,10 @@ def test_job_protocol_on_fake_runtime(tmp_path, algo, n_be, direct):
     if algo == "orion" and n_be > 0:
         masked = [b for b in res["launch_stream_masks"].values() if b > 0]
         assert masked and all(b in (32, 64, 128) for b in masked)
+    # hipMallocAsync / hipFreeAsync of every client: run by the client's own
+    # thread, on a stream the scheduler assigned (not the null stream they named)
+    assert sorted(t for s, t in res["async_allocs"]) == sorted(res["client_tids"])
+    assert sorted(t for s, t in res["async_frees"]) == sorted(res["client_tids"])
     for c in range(n_be):      # stopped early, not run to their 10000 iterations
         assert 0 < res["iters_done"][c] < 10_000
 
