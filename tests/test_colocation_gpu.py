@@ -42,6 +42,9 @@ def _check_replay(record_dir):
     elif seg[3] == "reef":
         from tests.test_policy_properties import check_reef_rule
         check_reef_rule(obs, jobs.native_replay(obs, by_poll=True))
+    elif seg[3] == "sequential":
+        from tests.test_policy_properties import check_time_slicing
+        check_time_slicing(obs, dec)
     return dec
 
 

@@ -268,6 +268,44 @@ def test_reef_rule_fires_every_branch(tmp_path):
     check_reef_rule(obs, jobs.native_replay(obs, by_poll=True))
 
 
+def check_time_slicing(obs_text, dec_text):
+    """Time slicing with the repaired rule: everything runs on client 0's stream
+    set (schedule_sequential, scheduler_eval.cpp:199-201, :225-227), and past the
+    tenth iteration a client's record -- other than an allocation -- goes out only
+    while no other client is in the middle of an iteration (the stated intent of
+    :189-196 and :213-221)."""
+    n = int(obs_text.split(" ", 2)[1])
+    seen, iters = [0] * n, [0] * n
+    exclusive = 0
+    for line in dec_text.splitlines():
+        p = line.split(" ")
+        if p[0] == "D":
+            c = int(p[1])
+            assert p[2] == "0", line
+            if n > 1 and iters[c] > 10 and p[3] != "m":
+                assert all(seen[j] == 0 for j in range(n) if j != c), (line, seen)
+                exclusive += 1
+            if p[3] == "k":
+                seen[c] += 1
+        elif p[0] == "F":
+            c = int(p[1])
+            seen[c], iters[c] = 0, iters[c] + 1
+    return exclusive
+
+
+@settings(max_examples=60, deadline=None,
+          suppress_health_check=[HealthCheck.function_scoped_fixture, HealthCheck.too_slow])
+@given(seed=st.integers(0, 10_000), n_clients=st.integers(1, 4), hp_iters=st.integers(12, 30))
+def test_time_slicing_never_overlaps_iterations(tmp_path_factory, seed, n_clients, hp_iters):
+    tmp = str(tmp_path_factory.mktemp("job"))
+    job = jobs.make_job(tmp, seed, n_clients=n_clients, algo=po.ALGO_SEQUENTIAL, hp_train=False,
+                        hp_iters=hp_iters)
+    _, _, rec = jobs.run_oracle(job)
+    dec = jobs.native_replay(rec.obs_text())
+    assert dec == rec.dec.text()
+    assert check_time_slicing(rec.obs_text(), dec) > 0 or n_clients == 1
+
+
 @settings(max_examples=150, deadline=None,
           suppress_health_check=[HealthCheck.function_scoped_fixture, HealthCheck.too_slow])
 @given(seed=st.integers(0, 10_000), n_clients=st.integers(1, 5),
