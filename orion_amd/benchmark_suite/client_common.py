@@ -8,14 +8,13 @@ bert_trainer_mock.py:49-234); the line numbers below are train_imagenet.py's.
 import json
 import os
 import random
+import threading
 import time
 
 import numpy as np
 import torch
 
 from .. import scheduler_frontend as fe
-
-import threading
 
 WARMUP_ITERS = 10     # iterations before the measured run (:188-198, :220)
 
@@ -85,6 +84,11 @@ def write_result(tid, data):
         json.dump(data, f)
 
 
+# Raised by the launcher's ``--algo streams`` baseline (no scheduler: nobody else
+# could tell the best-effort clients that the high-priority client is done).
+UNSCHEDULED_STOP = threading.Event()
+
+
 class Backend:
     """block()/stop() of libinttemp.so (:63-68, :88) plus stream registration."""
 
@@ -102,7 +106,7 @@ class Backend:
             torch.cuda.current_stream().synchronize()
 
     def stop(self):
-        return bool(self.lib.stop())
+        return bool(self.lib.stop()) or UNSCHEDULED_STOP.is_set()
 
     def register_stream(self, stream):
         self.lib.orion_register_stream(stream.cuda_stream)

@@ -42,6 +42,9 @@ def run_job(job, algo, workdir, max_be_duration, reef_depth=12, env=None,
     with open(cfg, "w") as f:
         json.dump(job, f, indent=1)
     e = preload_env({"ORION_RESULT_DIR": workdir, "ORION_QUIET": "1"})
+    if algo == "streams":      # the baseline without scheduler: no interception either
+        e["LD_PRELOAD"] = ":".join(p for p in e.get("LD_PRELOAD", "").split(":")
+                                   if p and p != _lib.CAPTURE_LIB)
     e.update(env or {})
     cmd = [sys.executable, "-u", "-m", "orion_amd.launch_jobs", "--algo", algo,
            "--config_file", cfg, "--orion_max_be_duration", str(max_be_duration),

@@ -101,7 +101,10 @@ def markdown(rows, figure):
 
 
 def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
-        experiment=None, fill_job=None, log=print):
+        experiment=None, fill_job=None, log=print, algo="orion"):
+    """``algo``: ``orion``, ``reef`` (depth 12), ``sequential``, or ``streams`` -- the
+    same clients on plain streams with no scheduler, the reference's "Streams"
+    baseline; it needs no profiles."""
     from . import colocate
     from .profiling import capture_profile
     experiment = experiment or colocate.experiment
@@ -112,7 +115,8 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
     if unknown:
         raise KeyError(f"unknown pairs {sorted(unknown)}; known: {sorted(todo)}")
     rows = []
-    with open(os.path.join(out_dir, f"fig{figure}.csv"), "w", newline="") as f:
+    suffix = "" if algo == "orion" else "_" + algo
+    with open(os.path.join(out_dir, f"fig{figure}{suffix}.csv"), "w", newline="") as f:
         writer = csv.DictWriter(f, fieldnames=FIELDS)
         writer.writeheader()
         for name, (job, budget) in todo.items():
@@ -123,9 +127,12 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
             cfg = os.path.join(base, "job.json")
             with open(cfg, "w") as jf:
                 json.dump(job, jf, indent=1)
-            filled = fill_job(cfg, os.path.join(base, "profiles"),
-                              os.path.join(base, "filled.json"), quiet=True)
-            res = experiment(filled, "orion", budget, base, repeats=repeats,
+            if algo == "streams":
+                filled = job
+            else:
+                filled = fill_job(cfg, os.path.join(base, "profiles"),
+                                  os.path.join(base, "filled.json"), quiet=True)
+            res = experiment(filled, algo, budget, base, repeats=repeats,
                              be_isolated_iters=60)
             row = row_of(name, budget, res, filled)
             writer.writerow(row)
@@ -133,7 +140,7 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
             rows.append(row)
             log(f"{name}: HP p99 x{row['hp_p99_ratio']:.2f}, BE keeps "
                 f"{100 * row['be_retained']:.0f} %")
-    with open(os.path.join(out_dir, f"fig{figure}.md"), "w") as f:
+    with open(os.path.join(out_dir, f"fig{figure}{suffix}.md"), "w") as f:
         f.write(markdown(rows, figure) + "\n")
     return rows
 
@@ -145,10 +152,13 @@ def main(argv=None):
     p.add_argument("--pairs", nargs="*", help="subset, e.g. rnet_rnet bert_mnet (BE_HP)")
     p.add_argument("--hp-requests", type=int, default=1200)
     p.add_argument("--repeats", type=int, default=2)
+    p.add_argument("--algo", default="orion",
+                   choices=["orion", "reef", "sequential", "streams"],
+                   help="policy, or streams: plain streams without a scheduler (baseline)")
     p.add_argument("--hp-trace", help="JSON list of inter-arrival times (s) for the "
                                       "high-priority client instead of Poisson arrivals")
     a = p.parse_args(argv)
-    rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace)
+    rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace, algo=a.algo)
     print(markdown(rows, a.figure))
 
 

@@ -73,9 +73,72 @@ def job_lists(config_dict_list):
     }
 
 
+class _UnscheduledRendezvous:
+    """``barriers[0]`` of the ``streams`` baseline.  Under the scheduler every
+    client meets the scheduler thread before it builds its model, after its
+    iterations 1 and 10, and at the end of its run; without one the clients meet
+    each other the first three times, and the fourth wait -- the end of a run --
+    returns at once, the high-priority client's after raising the stop flag the
+    best-effort clients poll."""
+
+    def __init__(self, num_clients):
+        self.barrier = threading.Barrier(num_clients)
+        self.hp_name = f"orion-client-{num_clients - 1}"
+        self.waits = {}
+
+    def wait(self):
+        me = threading.current_thread().name
+        self.waits[me] = self.waits.get(me, 0) + 1
+        if self.waits[me] <= 3:
+            self.barrier.wait()
+            return
+        if me == self.hp_name:
+            from .benchmark_suite import client_common
+            client_common.UNSCHEDULED_STOP.set()
+
+
+def launch_unscheduled(config_dict_list, function_dict=None):
+    """The clients as plain threads on streams of their own, no interception and
+    no scheduler: what the reference measures as its "streams" baseline with the
+    ``*_torch.py`` variants of its client loops
+    (benchmarking/benchmark_suite/train_imagenet_torch.py and siblings).  Same
+    loops, same result files."""
+    from .benchmark_suite.client_common import seed_everything
+    seed_everything(42)
+    function_dict = function_dict or _function_dict()
+    num_clients = len(config_dict_list)
+    rendezvous = _UnscheduledRendezvous(num_clients)
+    barriers = [rendezvous] * num_clients
+    client_barrier = threading.Barrier(num_clients)
+    threads, results = [], [None] * num_clients
+    for i, config_dict in enumerate(config_dict_list):
+        kwargs = dict(config_dict["args"])
+        kwargs.update({"num_iters": config_dict["num_iters"], "local_rank": 0,
+                       "barriers": barriers, "client_barrier": client_barrier, "tid": i})
+
+        def target(func=function_dict[config_dict["arch"]], kwargs=kwargs, i=i):
+            try:
+                results[i] = func(**kwargs)
+            except BaseException:
+                import traceback
+                traceback.print_exc()
+                print(f"orion: client {i} failed; aborting the job", flush=True)
+                os._exit(1)
+
+        thread = threading.Thread(target=target, name=f"orion-client-{i}")
+        thread.start()
+        threads.append(thread)
+    for thread in threads:
+        thread.join()
+    print("--------- all threads joined!", flush=True)
+    return results
+
+
 def launch_jobs(config_dict_list, input_args, run_eval=True, function_dict=None,
                 require_preload=True):
     """reference: launch_jobs.py:44-122."""
+    if getattr(input_args, "algo", None) == "streams":
+        return launch_unscheduled(config_dict_list, function_dict)
     from .benchmark_suite.client_common import seed_everything
     seed_everything(42)
     # All clients are threads of this interpreter and share its GIL.  The switch
@@ -143,7 +206,8 @@ def launch_jobs(config_dict_list, input_args, run_eval=True, function_dict=None,
 def build_parser():
     parser = argparse.ArgumentParser()
     parser.add_argument("--algo", type=str, required=False, default="orion",
-                        help="choose one of orion | reef | sequential")
+                        help="choose one of orion | reef | sequential (or streams: "
+                             "the clients on plain streams, no scheduler, as a baseline)")
     parser.add_argument("--config_file", type=str,
                         help="path to the experiment configuration file")
     parser.add_argument("--reef_depth", type=int, default=1,
@@ -167,8 +231,8 @@ def main(argv=None):
     if args.print_preload:
         print(_lib.CAPTURE_LIB)
         return 0
-    if args.algo not in ("orion", "reef", "sequential"):
-        raise SystemExit("--algo must be one of orion | reef | sequential")
+    if args.algo not in ("orion", "reef", "sequential", "streams"):
+        raise SystemExit("--algo must be one of orion | reef | sequential | streams")
     if not args.config_file:
         raise SystemExit("--config_file is required")
     import torch

@@ -178,3 +178,44 @@ def test_repeated_runs_are_pooled_request_by_request():
     # one run without the raw list (an older result file) keeps its own percentiles
     old = {k: v for k, v in a.items() if k != "latencies_ms"}
     assert colocate.pooled([old])["p99_latency"] == 1.0
+
+
+def test_streams_baseline_runs_the_same_loops_without_a_scheduler(tmp_path, monkeypatch):
+    """``--algo streams``: the clients rendezvous with each other after iterations
+    1 and 10, the high-priority client's end raises the stop flag, the best-effort
+    client stops at its next iteration; result files as under the scheduler."""
+    monkeypatch.setenv("ORION_RESULT_DIR", str(tmp_path))
+    cc.UNSCHEDULED_STOP.clear()
+    steps = {0: 0, 1: 0}
+
+    def loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank, barriers,
+             client_barrier, tid):
+        class NoGpu(cc.Backend):
+            def __init__(self):
+                pass
+
+            def block(self, it):
+                pass
+
+            def stop(self):
+                return cc.UNSCHEDULED_STOP.is_set()
+
+        def step(i):
+            steps[tid] += 1
+
+        barriers[0].wait()      # every client loop starts with this rendezvous
+        return cc.run_client(tid, train, num_iters, [0.0] * num_iters, barriers, step, NoGpu())
+
+    job = [{"arch": "x", "kernel_file": "", "num_kernels": 0, "num_iters": 10_000_000,
+            "args": {"batchsize": 1, "rps": 0, "uniform": False, "dummy_data": True,
+                     "train": True}},
+           {"arch": "x", "kernel_file": "", "num_kernels": 0, "num_iters": 60,
+            "args": {"batchsize": 1, "rps": 0, "uniform": False, "dummy_data": True,
+                     "train": False}}]
+    args = launch_jobs.build_parser().parse_args(["--algo", "streams", "--config_file", "x"])
+    res = launch_jobs.launch_jobs(job, args, function_dict={"x": loop})
+    cc.UNSCHEDULED_STOP.clear()
+    assert res[1]["iterations"] == 60 and steps[1] == 60
+    assert 10 <= res[0]["iterations"] < 10_000_000
+    assert json.load(open(tmp_path / "client_1.json"))["iterations"] == 60
+    assert "p99_latency" in res[1] and "throughput" in res[0]
