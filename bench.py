@@ -15,7 +15,9 @@ power-limited package needs to settle.  Prints ONE JSON line.
 Work done, in order (child processes first, so that this process has not touched
 the GPU when it starts them):
   1. profile both clients alone under the interception layer (gfx950 profiles);
-  2. high-priority client alone, best-effort client alone, both co-located;
+  2. high-priority client alone, best-effort client alone, both co-located
+     (then the same with a HIP-graph client, and once on plain streams with no
+     scheduler at all: `no_scheduler_baseline`);
   3. replay the recorded observation log through the CPU oracle and the native
      policy core: decision sequences must be identical;
   4. kernel pair in this process: GEMM and triad alone and side by side per
@@ -157,6 +159,8 @@ def main():
                          "starts no child process)")
     ap.add_argument("--no-hip-graph-leg", action="store_true",
                     help="skip the extra run with a HIP-graph high-priority client")
+    ap.add_argument("--no-streams-leg", action="store_true",
+                    help="skip the extra run of the pair on plain streams without scheduler")
     ap.add_argument("--pair-requests", type=int, default=300,
                     help="measured GEMM requests of the scheduled kernel pair")
     ap.add_argument("--repeats", type=int, default=3,
@@ -216,6 +220,19 @@ def main():
                 "be_colocated_iters_per_s": cg["be_colocated"][0]["throughput"],
                 "be_retained": cg["be_retained"][0],
                 "records_per_iteration": cg["num_kernels"]}
+        # The same pair with no scheduler and no interception (--algo streams):
+        # what the scheduler is for
+        if not args.no_streams_leg:
+            from orion_amd import colocate
+            job = c3_job(max(300, args.steps // 2) + 10)
+            sres = colocate.experiment(job, "streams", args.max_be_duration,
+                                       os.path.join(workdir, "streams"), be_isolated_iters=60)
+            out["no_scheduler_baseline"] = {
+                "isolated_ms": {k: sres["hp_isolated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
+                "colocated_ms": {k: sres["hp_colocated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
+                "p99_ratio": sres["hp_p99_ratio"],
+                "be_colocated_iters_per_s": sres["be_colocated"][0]["throughput"],
+                "be_retained": sres["be_retained"][0]}
         # configs[1] through the same hot path: GEMM requests (high priority)
         # beside the triad loop (best effort), default CU masks; back-to-back
         # requests (the high-priority client never idle) and Poisson arrivals
