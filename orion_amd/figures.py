@@ -50,9 +50,10 @@ def _entry(arch, model_name, batch, rps, uniform, train, num_iters, dtype, trace
             "args": args}
 
 
-def jobs(figure, hp_requests=1200, hp_trace=None):
+def jobs(figure, hp_requests=1200, hp_trace=None, hp_hip_graph=False):
     """name -> (job, duration budget): the last entry of a job is the
-    high-priority client, as the launcher expects."""
+    high-priority client, as the launcher expects.  ``hp_hip_graph``: the
+    high-priority client replays a captured HIP graph (one record per request)."""
     if figure not in (7, 10):
         raise ValueError("figure 7 (inference + training) or 10 (inference + inference)")
     out = {}
@@ -64,6 +65,8 @@ def jobs(figure, hp_requests=1200, hp_trace=None):
                 be = _entry(arch, model, inf_bs, inf_rps, True, False, 1_000_000, "bf16")
             hp = _entry(hp_arch, hp_arch, 4, 0 if hp_trace else hp_rps, False, False,
                         hp_requests + 10, "bf16", trace=hp_trace)
+            if hp_hip_graph:
+                hp["args"]["hip_graph"] = True
             out[f"{be_key}_{hp_key}"] = ([be, hp], budget)
     return out
 
@@ -101,7 +104,7 @@ def markdown(rows, figure):
 
 
 def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
-        experiment=None, fill_job=None, log=print, algo="orion"):
+        experiment=None, fill_job=None, log=print, algo="orion", hp_hip_graph=False):
     """``algo``: ``orion``, ``reef`` (depth 12), ``sequential``, or ``streams`` -- the
     same clients on plain streams with no scheduler, the reference's "Streams"
     baseline; it needs no profiles."""
@@ -110,12 +113,12 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
     experiment = experiment or colocate.experiment
     fill_job = fill_job or capture_profile.fill_job
     os.makedirs(out_dir, exist_ok=True)
-    todo = jobs(figure, -(-hp_requests // repeats), hp_trace)
+    todo = jobs(figure, -(-hp_requests // repeats), hp_trace, hp_hip_graph)
     unknown = set(pairs or []) - set(todo)
     if unknown:
         raise KeyError(f"unknown pairs {sorted(unknown)}; known: {sorted(todo)}")
     rows = []
-    suffix = "" if algo == "orion" else "_" + algo
+    suffix = ("" if algo == "orion" else "_" + algo) + ("_hip_graph" if hp_hip_graph else "")
     with open(os.path.join(out_dir, f"fig{figure}{suffix}.csv"), "w", newline="") as f:
         writer = csv.DictWriter(f, fieldnames=FIELDS)
         writer.writeheader()
@@ -155,10 +158,13 @@ def main(argv=None):
     p.add_argument("--algo", default="orion",
                    choices=["orion", "reef", "sequential", "streams"],
                    help="policy, or streams: plain streams without a scheduler (baseline)")
+    p.add_argument("--hp-hip-graph", action="store_true",
+                   help="the high-priority client replays a captured HIP graph per request")
     p.add_argument("--hp-trace", help="JSON list of inter-arrival times (s) for the "
                                       "high-priority client instead of Poisson arrivals")
     a = p.parse_args(argv)
-    rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace, algo=a.algo)
+    rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace, algo=a.algo,
+               hp_hip_graph=a.hp_hip_graph)
     print(markdown(rows, a.figure))
 
 
