@@ -80,3 +80,29 @@ def test_driver_writes_one_row_per_pair(tmp_path):
     assert rows[0]["pair"] == "rnet_rnet"
     with pytest.raises(KeyError):
         figures.run(7, str(tmp_path), pairs=["nope"], experiment=experiment, fill_job=fill_job)
+
+
+def test_hip_graph_and_other_policies_are_options_of_the_same_pairs(tmp_path):
+    plain = figures.jobs(7)
+    graph = figures.jobs(7, hp_hip_graph=True)
+    for name in plain:
+        assert graph[name][0][-1]["args"]["hip_graph"] is True
+        assert "hip_graph" not in plain[name][0][-1]["args"]
+        assert graph[name][0][0] == plain[name][0][0] and graph[name][1] == plain[name][1]
+    calls = []
+
+    def experiment(job, algo, budget, workdir, repeats, be_isolated_iters):
+        calls.append((algo, job[0]["num_kernels"]))
+        return {"hp_isolated": {"p50_latency": 1.0, "p99_latency": 2.0},
+                "hp_colocated": {"p50_latency": 1.0, "p99_latency": 2.0},
+                "hp_p50_ratio": 1.0, "hp_p99_ratio": 1.0,
+                "be_isolated": [{"throughput": 1.0}], "be_colocated": [{"throughput": 1.0}],
+                "be_retained": [1.0]}
+
+    def no_profiles(*a, **k):
+        raise AssertionError("the streams baseline needs no profiles")
+
+    figures.run(7, str(tmp_path), pairs=["rnet_rnet"], algo="streams", experiment=experiment,
+                fill_job=no_profiles, log=lambda *_: None)
+    assert calls == [("streams", 0)]
+    assert os.path.exists(tmp_path / "fig7_streams.csv") and os.path.exists(tmp_path / "fig7_streams.md")
