@@ -104,7 +104,8 @@ def markdown(rows, figure):
 
 
 def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
-        experiment=None, fill_job=None, log=print, algo="orion", hp_hip_graph=False):
+        experiment=None, fill_job=None, log=print, algo="orion", hp_hip_graph=False,
+        env=None):
     """``algo``: ``orion``, ``reef`` (depth 12), ``sequential``, or ``streams`` -- the
     same clients on plain streams with no scheduler, the reference's "Streams"
     baseline; it needs no profiles."""
@@ -135,8 +136,9 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
             else:
                 filled = fill_job(cfg, os.path.join(base, "profiles"),
                                   os.path.join(base, "filled.json"), quiet=True)
+            extra = {"env": dict(env)} if env else {}
             res = experiment(filled, algo, budget, base, repeats=repeats,
-                             be_isolated_iters=60)
+                             be_isolated_iters=60, **extra)
             row = row_of(name, budget, res, filled)
             writer.writerow(row)
             f.flush()
@@ -160,11 +162,13 @@ def main(argv=None):
                    help="policy, or streams: plain streams without a scheduler (baseline)")
     p.add_argument("--hp-hip-graph", action="store_true",
                    help="the high-priority client replays a captured HIP graph per request")
+    p.add_argument("--env", nargs="*", default=[], metavar="KEY=VALUE",
+                   help="environment of every run, e.g. ORION_MAX_SMS=8")
     p.add_argument("--hp-trace", help="JSON list of inter-arrival times (s) for the "
                                       "high-priority client instead of Poisson arrivals")
     a = p.parse_args(argv)
     rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace, algo=a.algo,
-               hp_hip_graph=a.hp_hip_graph)
+               hp_hip_graph=a.hp_hip_graph, env=dict(kv.split("=", 1) for kv in a.env))
     print(markdown(rows, a.figure))
 
 
