@@ -64,7 +64,7 @@ def _c3_job(hp_iters):
 
 
 def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_graph=False,
-               repeats=1):
+               repeats=1, extra_env=None):
     from orion_amd import colocate
     from orion_amd.profiling import capture_profile
     os.makedirs(workdir, exist_ok=True)
@@ -77,6 +77,7 @@ def colocation(steps, workdir, max_be_duration, masks, use_rocprof=False, hip_gr
     env = {"ORION_RECORD_DIR": os.path.join(workdir, "colocated")}
     if masks:
         env["ORION_BE_CU_MASKS"] = masks
+    env.update(extra_env or {})
     os.makedirs(env["ORION_RECORD_DIR"], exist_ok=True)
     res = colocate.experiment(job, "orion", max_be_duration, workdir, env=env, repeats=repeats)
     res["num_kernels"] = {"hp": job[-1]["num_kernels"],
@@ -212,8 +213,12 @@ def main():
         # schedules the request kernel by kernel.)
         if not args.no_hip_graph_leg:
             cg = colocation(max(300, args.steps // 2), os.path.join(workdir, "hip_graph"),
-                            args.max_be_duration, args.be_cu_masks, hip_graph=True)
+                            args.max_be_duration, args.be_cu_masks, hip_graph=True,
+                            extra_env={"ORION_RESERVE_HP_CUS": "1"})
             out["hp_hip_graph_variant"] = {
+                # the graph record needs every CU by profile; with this option the
+                # policy leaves best-effort kernels no room beside it
+                "options": {"ORION_RESERVE_HP_CUS": 1},
                 "isolated_ms": {k: cg["hp_isolated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
                 "colocated_ms": {k: cg["hp_colocated"][f"{k}_latency"] for k in ("p50", "p95", "p99")},
                 "p99_ratio": cg["hp_p99_ratio"],

@@ -15,8 +15,10 @@ Both logs are line-based text, shared with the native core
 (orion_amd/csrc/policy/obslog.h):
 
 observation log
-    ``J <n> <max_sms> <place_masks comma list> [L1]``   job header (L1: long
-                                                    best-effort kernels confined)
+    ``J <n> <max_sms> <place_masks comma list> [L1] [R1]``  job header (L1: long
+                                                    best-effort kernels confined; R1:
+                                                    the high-priority op's CU need
+                                                    is reserved)
     ``K <client> <num_kernels> <num_iters> <train 0|1> <profile path>``
     ``X <client> <num_kernels> <profile path>``      setup_change
     ``S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>``
@@ -99,10 +101,10 @@ class RecordingEnv(po.Env):
         self._dec = []
 
     # structure markers -------------------------------------------------
-    def header(self, max_sms, clients, confine_long=False):
+    def header(self, max_sms, clients, confine_long=False, reserve_hp=False):
         self.confine_long = bool(confine_long)
         self.obs.append(f"J {self.n} {max_sms} " + ",".join(map(str, self.masks))
-                        + (" L1" if confine_long else ""))
+                        + (" L1" if confine_long else "") + (" R1" if reserve_hp else ""))
         for i, (nk, ni, train, path) in enumerate(clients):
             self.obs.append(f"K {i} {nk} {ni} {int(bool(train))} {path}")
 
@@ -250,7 +252,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
     oracle = None
     rec = None
     n = max_sms = masks = None
-    confine_long = False
+    confine_long = reserve_hp = False
     clients = {}
     lines = obs_text.splitlines()
     i = 0
@@ -260,8 +262,9 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
         if tag == "J":
             n, max_sms = int(parts[1]), int(parts[2])
             masks = [int(x) for x in parts[3].split(",")]
-            _ensure(len(parts) == 4 or parts[4:] == ["L1"], "J: 3 fields and an optional L1")
-            confine_long = len(parts) == 5
+            _ensure(set(parts[4:]) <= {"L1", "R1"} and len(parts) <= 6,
+                    "J: 3 fields and optional L1 / R1")
+            confine_long, reserve_hp = "L1" in parts[4:], "R1" in parts[4:]
         elif tag == "K":
             clients[int(parts[1])] = (int(parts[2]), int(parts[3]),
                                       bool(int(parts[4])), " ".join(parts[5:]))
@@ -277,7 +280,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
                 oracle = po.PolicyOracle(
                     [load_profile(c[3]) for c in order], [c[0] for c in order],
                     [c[1] for c in order], [c[2] for c in order], max_sms,
-                    sequential_fix=sequential_fix)
+                    sequential_fix=sequential_fix, reserve_hp=reserve_hp)
             polls = []
             i += 1
             while lines[i] != "E":

@@ -157,7 +157,11 @@ class PolicyOracle:
     ``schedule`` calls: seen, event_ids, cur_iters, penalty, profiles."""
 
     def __init__(self, profiles, num_kernels, num_iters, is_train, max_sms=80,
-                 sequential_fix=False):
+                 sequential_fix=False, reserve_hp=False):
+        # reserve_hp (not in the reference): best-effort kernels admitted in one
+        # poll may add up to max_sms minus the CU need of the high-priority op
+        # last dispatched, instead of max_sms (:339 ignores that need).
+        self.reserve_hp = bool(reserve_hp)
         # sequential_fix: the reference's time-slicing policy can never
         # dispatch once a client is past its 10th iteration (see _sequential).
         # With the flag set, the evident intent is restated instead: dispatch
@@ -296,6 +300,7 @@ class PolicyOracle:
             sm_threshold = self.max_sms
             update_start = INT_MAX
         polls = 0
+        hp_need = 0
 
         while True:                                          # :277
             env.begin_poll()
@@ -316,6 +321,10 @@ class PolicyOracle:
                     op1 = self.ops[hp][self.seen[hp]]
                     self._dispatch(env, hp, hp, heads[hp])
                     profiles[hp] = op1.profile
+                    hp_need = op1.sm_used
+                room = sm_threshold
+                if self.reserve_hp and not self.is_train[hp]:
+                    room = max(0, sm_threshold - max(0, hp_need))
                 end = start + n                              # :323
                 for t in range(start + 1, end):
                     j = t % (n - 1)                          # :326
@@ -335,7 +344,7 @@ class PolicyOracle:
                           and env.event_done(hp, update_start - 1)):    # :338
                         go = True
                     elif (self.seen[hp] > 0
-                          and size + op0.sm_used <= sm_threshold
+                          and size + op0.sm_used <= room
                           and (op0.profile == -1 or profiles[hp] == -1
                                or profiles[hp] != op0.profile)):        # :340
                         go = True

@@ -20,11 +20,13 @@ void appendf(std::string* s, const char* fmt, ...) {
 }
 }  // namespace
 
-void Recorder::header(int max_sms, const std::vector<int>& masks, bool confine_long) {
+void Recorder::header(int max_sms, const std::vector<int>& masks, bool confine_long,
+                      bool reserve_hp) {
   appendf(&obs_, "J %d %d ", n_, max_sms);
   for (size_t i = 0; i < masks.size(); ++i)
     appendf(&obs_, i ? ",%d" : "%d", masks[i]);
   if (confine_long) obs_ += " L1";  // long best-effort kernels are confined
+  if (reserve_hp) obs_ += " R1";    // the high-priority op's CU need is reserved
   obs_ += '\n';
 }
 
@@ -231,7 +233,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
   };
 
   int n = 0, max_sms = 0;
-  bool confine_long = false;
+  bool confine_long = false, reserve_hp = false;
   std::vector<int> masks;
   std::vector<ClientDesc> clients;
   Policy* policy = nullptr;
@@ -245,12 +247,17 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
     if (l.empty()) continue;
     const char tag = l[0];
     if (tag == 'J') {
-      auto p = split(l, ' ', 5);
-      if (p.size() != 4 && !(p.size() == 5 && p[4] == "L1")) {
-        ok = bad(i, "J needs 3 fields and an optional L1");
+      auto p = split(l, ' ', 7);
+      bool options_ok = p.size() >= 4 && p.size() <= 6;
+      for (size_t k = 4; options_ok && k < p.size(); ++k) {
+        if (p[k] == "L1") confine_long = true;
+        else if (p[k] == "R1") reserve_hp = true;
+        else options_ok = false;
+      }
+      if (!options_ok) {
+        ok = bad(i, "J needs 3 fields and optional L1 / R1");
         break;
       }
-      confine_long = p.size() == 5;
       n = atoi(p[1].c_str());
       max_sms = atoi(p[2].c_str());
       for (auto& m : split(p[3], ',', 1u << 20)) masks.push_back(atoi(m.c_str()));
@@ -298,7 +305,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
         }
         if (!ok) break;
         policy = new Policy(std::move(profs), nk, ni, tr, max_sms, masks,
-                            sequential_fix, confine_long);
+                            sequential_fix, confine_long, reserve_hp);
       }
       ScheduleArgs a;
       a.warmup = atoi(p[1].c_str()) != 0;

@@ -38,7 +38,8 @@ class Recorder : public PolicyHost {
   // the decision log lines up with the observation log's P lines one to one.
   void set_mark_polls(bool on) { mark_polls_ = on; }
 
-  void header(int max_sms, const std::vector<int>& masks, bool confine_long = false);
+  void header(int max_sms, const std::vector<int>& masks, bool confine_long = false,
+              bool reserve_hp = false);
   void client(int idx, int num_kernels, int num_iters, bool train,
               const std::string& profile_path);
   void setup_change(int client, int num_kernels, const std::string& path);

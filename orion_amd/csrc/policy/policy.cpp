@@ -134,7 +134,8 @@ static int max_sm_used(const std::vector<OpInfo>& ops) {
 Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
                std::vector<int> num_kernels, std::vector<int> num_iters,
                std::vector<bool> is_train, int max_sms,
-               std::vector<int> cu_masks, bool sequential_fix, bool confine_long)
+               std::vector<int> cu_masks, bool sequential_fix, bool confine_long,
+               bool reserve_hp)
     : n_((int)profiles.size()),
       ops_(std::move(profiles)),
       num_kernels_(std::move(num_kernels)),
@@ -144,6 +145,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
       cu_masks_(std::move(cu_masks)),
       sequential_fix_(sequential_fix),
       confine_long_(confine_long),
+      reserve_hp_(reserve_hp),
       seen_(n_, 0),
       event_ids_(n_, 0),
       cur_iters_(n_, 0),
@@ -297,6 +299,7 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
   }
   std::vector<int> heads(n);
   int64_t polls = 0;
+  int hp_need = 0;  // CU need of the high-priority op last dispatched (reserve_hp_)
 
   for (;;) {
     host.begin_poll();
@@ -315,8 +318,14 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
     } else {
       if (heads[hp] != REC_NONE) {
         const int hp_profile = ops_[hp][seen_[hp]].profile;
+        hp_need = ops_[hp][seen_[hp]].sm_used;
         dispatch(host, hp, hp, heads[hp]);
         profiles[hp] = hp_profile;
+      }
+      int room = sm_threshold;
+      if (reserve_hp_ && !is_train_[hp]) {
+        room = sm_threshold - (hp_need > 0 ? hp_need : 0);
+        if (room < 0) room = 0;
       }
       const int end = start + n;
       for (int t = start + 1; t < end; ++t) {
@@ -333,7 +342,7 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
         } else if (seen_[hp] >= update_start && op0.sm_used <= sm_threshold &&
                    host.event_done(hp, update_start - 1)) {
           go = true;
-        } else if (seen_[hp] > 0 && size + op0.sm_used <= sm_threshold &&
+        } else if (seen_[hp] > 0 && size + op0.sm_used <= room &&
                    (op0.profile == -1 || profiles[hp] == -1 ||
                     profiles[hp] != op0.profile)) {
           go = true;

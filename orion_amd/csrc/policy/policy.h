@@ -108,7 +108,7 @@ class Policy {
          std::vector<int> num_kernels, std::vector<int> num_iters,
          std::vector<bool> is_train, int max_sms,
          std::vector<int> cu_masks, bool sequential_fix,
-         bool confine_long = false);
+         bool confine_long = false, bool reserve_hp = false);
 
   void setup_change(int client, std::vector<OpInfo> ops, int num_kernels);
 
@@ -142,6 +142,13 @@ class Policy {
   // Placement only: a best-effort kernel whose profiled duration alone exceeds
   // the duration budget is kept off the whole-GPU stream.
   bool confine_long_;
+  // Admission option (not in the reference, whose rule never looks at the
+  // high-priority op's own CU need, scheduler_eval.cpp:339): while a
+  // high-priority inference request is in flight, best-effort kernels admitted
+  // in one poll may add up to max_sms minus the CU need of the high-priority
+  // op last dispatched.  A whole-GPU op -- a HIP-graph request -- then leaves
+  // no room; short kernels with a small need leave nearly all of it.
+  bool reserve_hp_;
   // survive between schedule() calls, like the reference's globals
   std::vector<int> seen_;
   std::vector<int> event_ids_;

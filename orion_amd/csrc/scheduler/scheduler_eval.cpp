@@ -462,8 +462,11 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
   // budget off the whole-GPU stream even while the high-priority client is idle.
   const bool confine_long = getenv("ORION_CONFINE_LONG_BE") &&
                             atoi(getenv("ORION_CONFINE_LONG_BE")) != 0;
+  // Admission option: reserve the high-priority op's own CU need (see policy.h).
+  const bool reserve_hp = getenv("ORION_RESERVE_HP_CUS") &&
+                          atoi(getenv("ORION_RESERVE_HP_CUS")) != 0;
   g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, max_sms, g.masks,
-                            !as_written, confine_long));
+                            !as_written, confine_long, reserve_hp));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
   g.host->set_policy(g.policy.get());
   g.recorder.reset();
@@ -472,7 +475,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** /*models*/,
     if (*dir) {
       g.record_dir = dir;
       g.recorder.reset(new Recorder(g.host.get(), num_clients));
-      g.recorder->header(max_sms, g.masks, confine_long);
+      g.recorder->header(max_sms, g.masks, confine_long, reserve_hp);
       for (int i = 0; i < num_clients; ++i)
         g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
       // start both logs afresh

@@ -92,6 +92,7 @@ def make_job(tmp_path, seed, n_clients=2, algo=po.ALGO_ORION, hp_train=False,
     job.arrivals = [rng.randint(20_000, 2_000_000) for _ in range(16)]
     job.closed_loop_hp = rng.random() < 0.3 or hp_train
     job.confine_long = rng.random() < 0.5
+    job.reserve_hp = rng.random() < 0.4
     return job
 
 
@@ -99,7 +100,8 @@ def run_oracle(job, max_polls=3_000_000):
     profiles = [po.parse_profile(p) for p in job.paths]
     oracle = po.PolicyOracle(profiles, job.nk, job.iters, job.train,
                              max_sms=job.max_sms,
-                             sequential_fix=job.sequential_fix)
+                             sequential_fix=job.sequential_fix,
+                             reserve_hp=getattr(job, "reserve_hp", False))
     clients = []
     for c in range(job.n):
         first, main = job.traces[c]
@@ -117,7 +119,8 @@ def run_oracle(job, max_polls=3_000_000):
     rec.budget = job.depth
     rec.header(job.max_sms, [(job.nk[c], job.iters[c], job.train[c],
                               job.paths[c]) for c in range(job.n)],
-               confine_long=getattr(job, "confine_long", False))
+               confine_long=getattr(job, "confine_long", False),
+               reserve_hp=getattr(job, "reserve_hp", False))
     changes = {1: [(c, po.parse_profile(path), nk, path)
                    for c, (path, nk) in sorted(job.swap.items())]}
     vg.run_job(oracle, env, rec, [(True, 1), (True, 10), (False, 0)],

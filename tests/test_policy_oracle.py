@@ -171,6 +171,39 @@ def test_cu_budget_is_per_poll_and_round_robin_rotates():
     assert out[3] == [("D", 2, 2, K, 0, 0)]
 
 
+def test_reserving_the_high_priority_ops_own_cu_need():
+    """Not in the reference (its rule, :339, never reads cur_sms[hp]): with
+    reserve_hp the room for best-effort kernels in a poll is max_sms minus the CU
+    need of the high-priority op last dispatched.  max_sms = 80."""
+    hp = [op(0, 30, 100), op(0, 80, 100), op(0, 5, 100)]      # needs 30, 80, 5 CUs
+    be = [op(1, 40, 10)] * 9                                   # needs 40
+    heads = [{"heads": [K, K]}, {"heads": [K, K]},
+             {"heads": [K, K], "events": {(1, 2): False}}]   # third op ends the request
+    # as the reference: 40 <= 80 every time
+    o = make([be, hp], [9, 3], [100, 100], [True, False], cur_iters=[11, 11])
+    out = by_poll(run(o, [dict(h) for h in heads], depth=10**9))
+    assert [len(p) for p in out] == [2, 2, 3]
+    # reserved: room 80-30 = 50 -> admitted; 80-80 = 0 -> refused; 80-5 = 75 -> admitted
+    o = make([be, hp], [9, 3], [100, 100], [True, False], cur_iters=[11, 11], reserve_hp=True)
+    out = by_poll(run(o, [dict(h) for h in heads], depth=10**9))
+    assert out[0] == [("D", 1, 1, K, 0, 0), ("D", 0, 0, K, 0, 0)]
+    assert out[1] == [("D", 1, 1, K, 1, 1)]
+    assert out[2] == [("D", 1, 1, K, 2, 2), ("D", 0, 0, K, 1, 1), ("q", 1, 2)]
+    # the need stays reserved in polls without a new high-priority record, and
+    # goes when the request completes (seen[hp] == 0: everything is admitted)
+    hp2 = [op(0, 80, 100)] * 2
+    o = make([be, hp2], [9, 2], [100, 100], [True, False], cur_iters=[11, 11], reserve_hp=True)
+    out = by_poll(run(o, [
+        {"heads": [K, K]},                               # HP op needs 80: no room
+        {"heads": [K, None]},                            # still in flight: no room
+        {"heads": [K, K], "events": {(1, 1): True}},     # last HP op; request completes
+        {"heads": [K, None]},                            # idle: admitted
+    ], depth=10**9))
+    assert out[0] == [("D", 1, 1, K, 0, 0)] and out[1] == []
+    assert out[2] == [("D", 1, 1, K, 1, 1), ("q", 1, 1), ("F", 1, 11)]
+    assert out[3] == [("D", 0, 0, K, 0, 0)]
+
+
 def test_oversized_op_is_never_admitted_next_to_hp_but_runs_when_hp_idle():
     hp = [op(0, 10, 100)] * 2
     be = [op(1, 81, 10)] * 3          # needs more than max_sms = 80

@@ -337,11 +337,14 @@ def test_orion_invariants_on_recordings_of_the_live_scheduler(case):
 def test_the_checks_bite(tmp_path):
     """The invariants are not vacuous: every kind fires on an ordinary job, and a
     log with one best-effort dispatch moved to the neighbouring poll fails."""
-    job = jobs.make_job(str(tmp_path), 11, n_clients=3, hp_iters=25, depth=150_000)
-    _, _, rec = jobs.run_oracle(job)
-    obs = rec.obs_text()
-    marked = jobs.native_replay(obs, by_poll=True)
-    counts = check_orion_invariants(obs, marked, 150_000)
+    counts = {}
+    for seed in range(11, 17):
+        job = jobs.make_job(str(tmp_path), seed, n_clients=3, hp_iters=25, depth=150_000)
+        _, _, rec = jobs.run_oracle(job)
+        obs = rec.obs_text()
+        marked = jobs.native_replay(obs, by_poll=True)
+        for k, v in check_orion_invariants(obs, marked, 150_000).items():
+            counts[k] = counts.get(k, 0) + v
     assert all(v > 0 for v in counts.values()), counts
     lines = marked.splitlines()
     # move the first high-priority dispatch one poll later
