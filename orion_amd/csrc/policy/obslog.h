@@ -9,7 +9,9 @@
 //
 // Line formats (text, one record per line):
 //   observation log
-//     J <n> <max_sms> <cu mask sizes, comma separated>
+//     J <n> <max_sms> <cu mask sizes, comma separated> [L1] [R1]
+//       (L1: long best-effort kernels are confined to a partial mask;
+//        R1: the high-priority op's own CU need is reserved)
 //     K <client> <num_kernels> <num_iters> <train 0|1> <profile path>
 //     X <client> <num_kernels> <profile path>               setup_change
 //     S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>
