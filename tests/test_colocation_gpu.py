@@ -324,12 +324,14 @@ def test_hip_graph_replays_match_eager_every_time(dtype, tol):
             _ = (x.cuda() * 2).sum().item()          # eager work between replays
 
 
-@pytest.mark.parametrize("direct", ["1", "0"])
-def test_hip_graph_client_beside_a_trainer(tmp_path, direct):
+@pytest.mark.parametrize("direct,reserve", [("1", "0"), ("0", "0"), ("1", "1")])
+def test_hip_graph_client_beside_a_trainer(tmp_path, direct, reserve):
     """A launch-bound inference client that replays a captured HIP graph: one
     copy record and one hipGraphLaunch record per request through the same hot
     path, beside a best-effort trainer -- issued by the client itself (default)
-    or handed to the scheduler thread (ORION_HP_DIRECT=0)."""
+    or handed to the scheduler thread (ORION_HP_DIRECT=0); once with the policy
+    reserving the graph record's CU need (ORION_RESERVE_HP_CUS=1), which the
+    log header records and the replays follow."""
     job = [
         {"arch": "resnet50", "kernel_file": "", "num_kernels": 0, "num_iters": 100000,
          "args": {"model_name": "resnet50", "batchsize": 8, "rps": 0, "uniform": False,
@@ -339,7 +341,10 @@ def test_hip_graph_client_beside_a_trainer(tmp_path, direct):
                   "dummy_data": True, "train": False, "dtype": "fp32", "hip_graph": True}},
     ]
     filled, co, iso_out, co_out, co_dir = _run_iso_and_co(
-        str(tmp_path), job, extra_env={"ORION_HP_DIRECT": direct})
+        str(tmp_path), job, extra_env={"ORION_HP_DIRECT": direct,
+                                       "ORION_RESERVE_HP_CUS": reserve})
+    header = open(os.path.join(co_dir, "observations.log")).readline().split()
+    assert ("R1" in header) == (reserve == "1")
     assert filled[-1]["num_kernels"] == 1           # the graph is one record
     assert open(filled[-1]["kernel_file"]).read().splitlines()[1].startswith("hipGraphLaunch,-1,0,256,")
     assert co[-1]["iterations"] == 60 and co[0]["iterations"] >= 10
