@@ -20,6 +20,8 @@ req/s on average); pass it with ``--hp-trace`` to do the same.
     driver starts with the interception library preloaded.
 
     python -m orion_amd.figures --figure 7 --out fig7 [--pairs rnet_rnet bert_mnet]
+        [--algo orion|reef|sequential|streams] [--hp-hip-graph]
+        [--env ORION_RESERVE_HP_CUS=1 ...] [--hp-trace inter_arrival_times.json]
 """
 
 import argparse
