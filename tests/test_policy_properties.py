@@ -21,7 +21,9 @@ bookkeeping (seen[], iteration counts, the running best-effort duration sum):
   fits the CU budget of this poll and is of the opposite (or unknown) class
   (:339);
 * once the running sum of profiled durations exceeds the budget nothing
-  best-effort goes out until a poll that queried events (:341-357, :363-367).
+  best-effort goes out until a poll that queried events (:341-357, :363-367);
+* (this build's recorded option R1) the room of the CU budget is what the
+  high-priority op last dispatched leaves of it.
 
 Profile durations are whole numbers below 2^24, so the reference's float/long
 sum is exact here.
@@ -70,6 +72,8 @@ def check_orion_invariants(obs_text, dec_text, depth):
         if p[0] == "J":
             n, max_sms = int(p[1]), int(p[2])
             hp = n - 1
+            reserve_hp = "R1" in p[4:]      # this build's option: see below
+            hp_need = 0
         elif p[0] == "K":
             c = int(p[1])
             nk[c], max_iters[c], prof[c] = int(p[2]), int(p[3]), rows_of(p[5])
@@ -113,6 +117,7 @@ def check_orion_invariants(obs_text, dec_text, depth):
                 row = prof[c][op] if op < len(prof[c]) else None
                 if c == hp:
                     hp_profile = row[0] if row else None
+                    hp_need = max(0, row[1]) if row else 0
                     if cls == "k":        # only kernel records advance either counter
                         seen[c] += 1      # (utils_sched.cpp:240-249 against :251-282)
                         event_ids[c] += 1
@@ -129,6 +134,9 @@ def check_orion_invariants(obs_text, dec_text, depth):
                              or hp_done)
                 if not free_pass and row is not None and hp_profile is not None:
                     assert size + row[1] <= max_sms, (line, b, size)
+                    if reserve_hp:      # the HP op's own CU need is taken out of the room
+                        assert size + row[1] <= max(0, max_sms - hp_need), (line, b, hp_need)
+                        checked["reserved"] = checked.get("reserved", 0) + 1
                     assert row[0] == -1 or hp_profile == -1 or row[0] != hp_profile, (line, b)
                     checked["budget"] += 1
                 if row is not None:
