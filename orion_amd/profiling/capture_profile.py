@@ -134,7 +134,11 @@ def capture(entry, out_prefix, iters=14, function_dict=None):
 def profile_name(entry):
     a = entry["args"]
     phase = "train" if a["train"] else "inf"
-    return f"{a.get('model_name', entry['arch'])}_{a['batchsize']}_{a.get('dtype', 'fp32')}_{phase}"
+    # a HIP-graph client submits one record where the eager one submits hundreds:
+    # the two must not share a profile
+    graph = "_hipgraph" if a.get("hip_graph") else ""
+    return (f"{a.get('model_name', entry['arch'])}_{a['batchsize']}_{a.get('dtype', 'fp32')}_"
+            f"{phase}{graph}")
 
 
 def fill_job(config_path, out_dir, filled_path, iters=14, quiet=False, use_rocprof=False):

@@ -141,3 +141,18 @@ def test_trace_summary_cuts_requests_from_the_end(tmp_path):
     assert s["77"]["span_ms"]["p50"] == 0.007        # 6 us of kernels + two 0.5 us gaps
     assert abs(s["77"]["sum_ms"] - (0.11 + 100 * 0.006)) < 1e-9
     assert s["88"] == {"kernels": 5, "sum_ms": 35 / 1e6, "mean_us": 0.007, "queues": [4]}
+
+
+def test_profile_names_keep_clients_apart():
+    """Two clients of one job share a profile only when they submit the same
+    records: a HIP-graph client (one record per request) and the eager client of
+    the same model, batch and dtype do not."""
+    from orion_amd.profiling import capture_profile as cp
+    eager = {"arch": "resnet50", "args": {"model_name": "resnet50", "batchsize": 4,
+                                          "dtype": "bf16", "train": False}}
+    graph = {"arch": "resnet50", "args": dict(eager["args"], hip_graph=True)}
+    train = {"arch": "resnet50", "args": dict(eager["args"], train=True)}
+    names = {cp.profile_name(e) for e in (eager, graph, train)}
+    assert len(names) == 3 and cp.profile_name(eager) == "resnet50_4_bf16_inf"
+    assert cp.profile_name({"arch": "bert", "args": {"batchsize": 8, "train": True}}) == \
+        "bert_8_fp32_train"
