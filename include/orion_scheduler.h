@@ -118,13 +118,15 @@ void orion_thread_passthrough(int on);
 
 /* No reference counterpart: how many records `client` has queued since the job
  * was set up, and how many of them it queued without waiting for their
- * dispatch.  The latter is zero unless ORION_BE_RUN_AHEAD=1 is set: then a
- * best-effort client's kernel launches, device-to-device copies and fills are
- * queued with a deep copy of their arguments and the call returns at once
+ * dispatch.  The latter is zero unless ORION_BE_RUN_AHEAD=1 is set and setup()
+ * was given "gemm_bf16" or "triad_f32" as the client's model name (clients made
+ * of this library's own kernels; no other client is ever cleared for it): then
+ * the best-effort client's kernel launches, device-to-device copies and fills
+ * are queued with a deep copy of their arguments and the call returns at once
  * (hipSuccess, as every queued call of the reference returns:
  * intercept_temp.cpp:418-458), up to 64 records ahead of the scheduler.  By
- * default every record is handed over synchronously, as in the reference
- * (intercept_temp.cpp:404-416). */
+ * default, and for every other client always, every record is handed over
+ * synchronously, as in the reference (intercept_temp.cpp:404-416). */
 unsigned long long orion_client_submitted(int client);
 unsigned long long orion_client_deferred(int client);
 

@@ -158,6 +158,9 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
     scheduler on ``barriers[0]`` after iterations 1 and 10 and once at the end.
     """
     timings = []
+    # ORION_CLIENT_STAMPS=1: per request, how long the client spent submitting
+    # (inside step) and how long waiting for completion (inside block)
+    stamps = [] if os.environ.get("ORION_CLIENT_STAMPS", "0") not in ("", "0") else None
     batch_idx = 0
     start = time.time()
     next_startup = time.time()
@@ -178,9 +181,14 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
         else:
             if time.time() < next_startup:
                 continue
+            t_begin = time.time()
             step(batch_idx)
+            t_submitted = time.time()
             backend.block(batch_idx)
-            timings.append(time.time() - next_startup)
+            t_done = time.time()
+            timings.append(t_done - next_startup)
+            if stamps is not None:
+                stamps.append((t_begin - next_startup, t_submitted - t_begin, t_done - t_submitted))
             if batch_idx >= WARMUP_ITERS and sleep_times[batch_idx] > 0:
                 next_startup += sleep_times[batch_idx]
             else:
@@ -209,5 +217,8 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
         # every measured request, in arrival order (the reference's file holds
         # the percentiles only): lets runs be pooled
         data["latencies_ms"] = [round(float(t) * 1000, 4) for t in timings[drop:]]
+        if stamps is not None:
+            for k, name in enumerate(("start_delay_ms", "submit_ms", "wait_ms")):
+                data[name] = [round(float(s[k]) * 1000, 4) for s in stamps[drop:]]
     write_result(tid, data)
     return data

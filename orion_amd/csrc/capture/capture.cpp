@@ -308,20 +308,27 @@ void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_ti
     ch.direct_stream.store(nullptr);
     ch.submitted.store(0);
     ch.block_calls.store(0);
+    ch.may_run_ahead.store(0);
     // own_streams survive: a client may register its stream before setup runs
   }
-  // Off unless asked for: with it on, a ResNet-50 trainer beside a ResNet-50
-  // inference client has faulted an MI355X, cause not found (the hand-written
-  // kernel pair runs with it, bit-exact).  The two ways a launch is made
-  // self-contained can be told apart: ORION_BE_RUN_AHEAD_HOLDERS=0 leaves
-  // hipLaunchKernel synchronous (no graph kernel nodes), so that only module
-  // launches with one argument buffer, device copies and fills are queued ahead.
+  // Off unless asked for, and then only for the clients the scheduler clears
+  // afterwards (orion_capture_allow_run_ahead): with a ResNet-50 trainer queueing
+  // ahead beside a ResNet-50 inference client an MI355X has faulted, cause not
+  // found, so no framework client is ever cleared (the hand-written kernel pair
+  // runs with it, bit-exact).  On the host-only stand-in runtime the tests can
+  // leave hipLaunchKernel synchronous (ORION_BE_RUN_AHEAD_HOLDERS=0), which takes
+  // the graph kernel nodes out of the picture.
   const char* ahead = getenv("ORION_BE_RUN_AHEAD");
-  const char* holders = getenv("ORION_BE_RUN_AHEAD_HOLDERS");
+  const char* holders = orion_hip_api()->stand_in ? getenv("ORION_BE_RUN_AHEAD_HOLDERS") : nullptr;
   g_state.run_ahead.store(ahead && atoi(ahead) != 0 ? 1 : 0, std::memory_order_release);
   g_state.run_ahead_holders.store(holders && atoi(holders) == 0 ? 0 : 1, std::memory_order_release);
   g_state.epoch.fetch_add(1, std::memory_order_acq_rel);
   g_state.armed.store(1, std::memory_order_release);
+}
+
+void orion_capture_allow_run_ahead(int client, int allow) {
+  if (client < 0 || client >= kMaxClients) return;
+  g_state.channels[client].may_run_ahead.store(allow ? 1 : 0, std::memory_order_release);
 }
 
 void orion_capture_disarm(void) {
@@ -443,6 +450,12 @@ double stuck_limit_s() {
   return limit;
 }
 
+double monotonic_s() {
+  timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
 // Gives a record a deep copy of everything it points to, so that it can wait in
 // the queue after the call that made it has returned.  Returns false when the
 // record cannot be made self-contained (then the caller waits for its dispatch,
@@ -487,19 +500,24 @@ bool make_self_contained(ClientChannel& ch, uint32_t slot_index, Record& r) {
       p.blockDim = to_dim3(r.u.launch.block);
       p.sharedMemBytes = (unsigned int)r.u.launch.shmem;
       p.kernelParams = r.u.launch.args;
-      if (aux.holder && hip->hipGraphKernelNodeSetParams(aux.holder, &p) != hipSuccess) {
-        // A node does not take every kernel: the runtime checks the new block
-        // against the launch bounds of the kernel the node holds and answers
-        // hipErrorLaunchFailure when that one's are smaller.  Start afresh.
-        (void)hip->hipGetLastError();
+      // A node keeps the kernel it was created for: the runtime checks new
+      // parameters against the launch bounds of the kernel the node *holds*
+      // (hipErrorLaunchFailure when that one's are smaller than the new block),
+      // so nothing it does with a node that changes kernels is relied on here.
+      // Another kernel through this slot gets a fresh node.
+      if (aux.holder && (aux.holder_func != r.u.launch.func ||
+                         hip->hipGraphKernelNodeSetParams(aux.holder, &p) != hipSuccess)) {
+        if (aux.holder_func == r.u.launch.func) (void)hip->hipGetLastError();
         if (hip->hipGraphDestroyNode) (void)hip->hipGraphDestroyNode(aux.holder);
         aux.holder = nullptr;
       }
-      if (!aux.holder &&
-          hip->hipGraphAddKernelNode(&aux.holder, ch.holder_graph, nullptr, 0, &p) != hipSuccess) {
-        aux.holder = nullptr;
-        (void)hip->hipGetLastError();   // the real launch will tell the caller what is wrong
-        return false;
+      if (!aux.holder) {
+        if (hip->hipGraphAddKernelNode(&aux.holder, ch.holder_graph, nullptr, 0, &p) != hipSuccess) {
+          aux.holder = nullptr;
+          (void)hip->hipGetLastError();   // the real launch will tell the caller what is wrong
+          return false;
+        }
+        aux.holder_func = r.u.launch.func;
       }
       hipKernelNodeParams owned = {};
       if (hip->hipGraphKernelNodeGetParams(aux.holder, &owned) != hipSuccess ||
@@ -517,12 +535,16 @@ bool make_self_contained(ClientChannel& ch, uint32_t slot_index, Record& r) {
       const void* buffer = nullptr;
       const size_t* size = nullptr;
       void** e = r.u.module.extra;
-      for (int i = 0; i < 6 && e[i] != HIP_LAUNCH_PARAM_END; i += 2) {
-        if (e[i] == HIP_LAUNCH_PARAM_BUFFER_POINTER) buffer = e[i + 1];
-        else if (e[i] == HIP_LAUNCH_PARAM_BUFFER_SIZE) size = (const size_t*)e[i + 1];
+      // exactly {POINTER, buffer, SIZE, &size, END}, in either order: anything
+      // else (a longer list, a tag this code does not know) is left to the caller
+      int i = 0;
+      for (; i < 4 && e[i] != HIP_LAUNCH_PARAM_END; i += 2) {
+        if (e[i] == HIP_LAUNCH_PARAM_BUFFER_POINTER && !buffer) buffer = e[i + 1];
+        else if (e[i] == HIP_LAUNCH_PARAM_BUFFER_SIZE && !size) size = (const size_t*)e[i + 1];
         else return false;
       }
-      if (!buffer || !size || *size > kInlineKernarg) return false;
+      if (e[i] != HIP_LAUNCH_PARAM_END) return false;
+      if (!buffer || !size || *size == 0 || *size > kInlineKernarg) return false;
       memcpy(aux.kernarg, buffer, *size);
       aux.kernarg_size = *size;
       aux.extra[0] = HIP_LAUNCH_PARAM_BUFFER_POINTER;
@@ -574,6 +596,11 @@ void flush_channel(ClientChannel& ch) {
       continue;
     }
     if (rec->status != kRecordDeferred) break;
+    // Between two phases of a job a kernel stays where it is: the policy counts
+    // every kernel record against the client's profile rows, and one issued
+    // here would be missing from that count.  The scheduler takes it when it is
+    // back in its loop; copies and fills, which the policy does not count, go.
+    if (armed && rec_class_of(rec->type) == REC_KERNEL) break;
     hipStream_t stream = armed ? ch.last_stream.load(std::memory_order_acquire) : nullptr;
     if (stream == nullptr) stream = named_stream(*rec);
     ++tl_bypass;
@@ -591,11 +618,30 @@ void flush_channel(ClientChannel& ch) {
 // issued client idx's queue up to ticket `upto`.
 void wait_issued_upto(ClientChannel& ch, uint64_t upto) {
   unsigned spins = 0;
+  unsigned long waited = 0;
+  double idle_since = 0.0;
   while (ch.head.load(std::memory_order_acquire) < upto) {
     if (!g_state.armed.load(std::memory_order_acquire) ||
         !g_state.scheduler_polling.load(std::memory_order_acquire))
       flush_channel(ch);
-    if (ch.head.load(std::memory_order_acquire) < upto) cpu_relax(spins);
+    if (ch.head.load(std::memory_order_acquire) >= upto) break;
+    cpu_relax(spins);
+    // a kernel queued while the scheduler is between two phases stays queued
+    // (flush_channel leaves it to the policy); if the scheduler never comes
+    // back for it, say so instead of spinning forever
+    if ((++waited & 0xfffff) != 0) continue;
+    if (g_state.scheduler_polling.load(std::memory_order_acquire)) {
+      idle_since = 0.0;
+      continue;
+    }
+    const double now = monotonic_s();
+    if (idle_since == 0.0) idle_since = now;
+    if (now - idle_since > stuck_limit_s()) {
+      fprintf(stderr, "orion: a client has waited %.0f s for records it queued ahead while the "
+                      "scheduler is not polling; its iteration probably holds more kernel "
+                      "records than its profile's num_kernels\n", now - idle_since);
+      abort();
+    }
   }
 }
 
@@ -681,7 +727,8 @@ bool postpone_release(int kind, void* what) {
   if (!g_state.armed.load(std::memory_order_acquire) ||
       !g_state.run_ahead.load(std::memory_order_acquire) || tl_bypass)
     return false;
-  run_postponed(false);
+  // each release waits for the device: never on the high-priority client's thread
+  if (tl_client != g_state.num_clients - 1) run_postponed(false);
   Postponed p;
   p.kind = kind;
   p.what = what;
@@ -730,7 +777,7 @@ int submit(int idx, Record& r, bool wait) {
   const uint32_t slot_index = (uint32_t)(ticket & (kQueueSlots - 1));
   Record* slot = &ch.slots[slot_index];
   r.status = 0;
-  r.sync_stream = nullptr;
+  r.cell = nullptr;
   if (hipStream_t direct = ch.direct_stream.load(std::memory_order_acquire)) {
     // The scheduler lets this client issue its own calls: run the call here, on
     // the stream the scheduler named, under the producer lock so that the
@@ -749,6 +796,7 @@ int submit(int idx, Record& r, bool wait) {
       ch.last_stream.store(direct, std::memory_order_release);
     slot->type = r.type;
     slot->status = kRecordIssued;
+    slot->cell = nullptr;
     ch.tail.store(ticket + 1, std::memory_order_release);
     ch.submitted.store(ch.submitted.load(std::memory_order_relaxed) + 1, std::memory_order_relaxed);
     ch.producer_lock.store(0, std::memory_order_release);
@@ -756,8 +804,15 @@ int submit(int idx, Record& r, bool wait) {
   }
   const bool deferred = wait && idx < g_state.num_clients - 1 &&
                         g_state.run_ahead.load(std::memory_order_relaxed) &&
+                        ch.may_run_ahead.load(std::memory_order_relaxed) &&
                         make_self_contained(ch, slot_index, r);
+  // The outcome of a record its caller waits for comes back through storage of
+  // this call, never through the slot: once the scheduler has retired the record
+  // the slot is free, and another thread of this client (an autograd worker, a
+  // thread launching ahead) may already be writing ticket + kQueueSlots into it.
+  WaitCell cell = {kRecordPending, nullptr};
   if (deferred) r.status = kRecordDeferred;
+  else if (wait) r.cell = &cell;
   *slot = r;
   ch.tail.store(ticket + 1, std::memory_order_release);
   ch.submitted.store(ch.submitted.load(std::memory_order_relaxed) + 1, std::memory_order_relaxed);
@@ -787,9 +842,7 @@ int submit(int idx, Record& r, bool wait) {
       if (g_state.scheduler_polling.load(std::memory_order_acquire)) {
         idle_since = 0.0;
       } else {
-        timespec ts;
-        clock_gettime(CLOCK_MONOTONIC, &ts);
-        const double now = (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+        const double now = monotonic_s();
         if (idle_since == 0.0) idle_since = now;
         if (now - idle_since > stuck_limit_s()) {
           fprintf(stderr,
@@ -800,10 +853,43 @@ int submit(int idx, Record& r, bool wait) {
         }
       }
     }
+    if (!g_state.scheduler_polling.load(std::memory_order_acquire) &&
+        g_state.armed.load(std::memory_order_acquire) && rec_class_of(r.type) != REC_KERNEL) {
+      // Between two phases of a job nobody polls, and the scheduler thread will
+      // not be back before this client has reached the rendezvous (a copy that
+      // reads a result back after the last kernel of a warm-up iteration: the
+      // reference's caller would spin forever, intercept_temp.cpp:404-416).  A
+      // record the policy does not count is run here, in order, where the
+      // client's latest record went -- under the flush lock, through which the
+      // scheduler passes after raising scheduler_polling on its way back in, so
+      // that exactly one of the two runs it.
+      flush_channel(ch);   // records queued ahead of this one that nobody waits for
+      unsigned lock_spins = 0;
+      while (ch.flush_lock.exchange(1)) cpu_relax(lock_spins);
+      const bool mine = !g_state.scheduler_polling.load() && g_state.armed.load() &&
+                        ch.head.load(std::memory_order_acquire) == ticket;
+      int st = 0;
+      if (mine) {
+        hipStream_t stream = ch.last_stream.load(std::memory_order_acquire);
+        if (stream == nullptr) stream = named_stream(r);
+        if (orion_record_runs_on_caller(r.type)) {
+          st = execute_on_caller(r, stream);
+        } else {
+          ++tl_bypass;
+          st = orion_execute_record(&r, stream);
+          --tl_bypass;
+        }
+        ch.head.store(ticket + 1, std::memory_order_release);
+      }
+      ch.flush_lock.store(0);
+      if (mine) return st;
+    }
     if (!g_state.armed.load(std::memory_order_acquire)) {
       // The scheduler has left its loop for good.  Whatever it did not take is
       // run here, in order, on the stream the call named: first the records
-      // queued ahead of this one that nobody waits for, then this one.
+      // queued ahead of this one that nobody waits for, then this one.  (The
+      // slot still holds this record while head == ticket: nothing can be
+      // written over a record that has not been retired.)
       flush_channel(ch);
       if (ch.head.load(std::memory_order_acquire) > ticket) break;
       if (ch.head.load(std::memory_order_acquire) < ticket) {
@@ -811,11 +897,11 @@ int submit(int idx, Record& r, bool wait) {
         continue;
       }
       int st;
-      if (orion_record_runs_on_caller(slot->type)) {
-        st = execute_on_caller(*slot, named_stream(*slot));
+      if (orion_record_runs_on_caller(r.type)) {
+        st = execute_on_caller(r, named_stream(r));
       } else {
         ++tl_bypass;
-        st = orion_execute_record(slot, named_stream(*slot));
+        st = orion_execute_record(&r, named_stream(r));
         --tl_bypass;
       }
       ch.head.store(ticket + 1, std::memory_order_release);
@@ -823,9 +909,15 @@ int submit(int idx, Record& r, bool wait) {
     }
     cpu_relax(spins);
   }
-  if (slot->status == ORION_GRANTED_TO_CALLER)
-    return execute_on_caller(r, slot->sync_stream);
-  return slot->status;
+  // the scheduler wrote the cell before it moved head past the ticket
+  if (cell.status == kRecordPending) {
+    fprintf(stderr, "orion: client %d: record %llu (type %d) was retired without an outcome\n",
+            idx, (unsigned long long)ticket, r.type);
+    abort();
+  }
+  if (cell.status == ORION_GRANTED_TO_CALLER)
+    return execute_on_caller(r, cell.sync_stream);
+  return cell.status;
 }
 
 // Stream a client-side wait or event record is redirected to: where the
@@ -949,15 +1041,26 @@ hipError_t hipMalloc(void** ptr, size_t size) {
   const int idx = client_for_call(nullptr);
   if (idx < 0) return orion_hip_api()->hipMalloc(ptr, size);
   if (g_state.run_ahead.load(std::memory_order_acquire)) {
-    run_postponed(false);
+    // postponed releases wait for the device: not on the high-priority client
+    if (idx < g_state.num_clients - 1) run_postponed(false);
     // An allocation is ordered against nothing, and its caller may hold a lock
     // the high-priority client needs (a caching allocator calls it under its
     // own): it must not wait behind records queued ahead, whose turn depends on
     // that client's progress.  With nothing queued it is a record like any
     // other, which every policy dispatches in the poll that sees it.
     ClientChannel& ch = g_state.channels[idx];
-    if (ch.head.load(std::memory_order_acquire) < ch.deferred_upto.load(std::memory_order_acquire))
-      return orion_hip_api()->hipMalloc(ptr, size);
+    if (ch.head.load(std::memory_order_acquire) < ch.deferred_upto.load(std::memory_order_acquire)) {
+      hipError_t err = orion_hip_api()->hipMalloc(ptr, size);
+      if (err == hipErrorOutOfMemory && g_postponed_count.load(std::memory_order_acquire) > 0) {
+        // memory the caller believes free may still be held by postponed
+        // releases: carry out the ones whose queues have moved on and try once
+        // more (waiting for the others could wait for this very caller)
+        (void)orion_hip_api()->hipGetLastError();
+        run_postponed(false);
+        err = orion_hip_api()->hipMalloc(ptr, size);
+      }
+      return err;
+    }
   }
   Record r;
   r.type = RT_MALLOC;

@@ -6,12 +6,15 @@
 // then block() spins until the queue is empty), which is also what keeps
 // `void** args` -- pointers into the caller's frame -- alive until the launch.
 // Here that is the default as well.  With ORION_BE_RUN_AHEAD=1 it holds only for
-// the high-priority client and for every call whose result the caller needs: a
-// best-effort client's kernel launches, device-to-device copies and fills are
-// then queued with a deep copy of their arguments and the caller goes on at
-// once (up to kQueueSlots records ahead), so that when the policy lets
-// best-effort work in again after a pause the next records are already waiting
-// instead of being produced one by one at the client's own pace.
+// the high-priority client, for every call whose result the caller needs, and
+// for every client the scheduler has not cleared for it (see
+// orion_capture_allow_run_ahead: only clients made of this library's own
+// kernels are cleared; a framework model never is): a cleared best-effort
+// client's kernel launches, device-to-device copies and fills are then queued
+// with a deep copy of their arguments and the caller goes on at once (up to
+// kQueueSlots records ahead), so that when the policy lets best-effort work in
+// again after a pause the next records are already waiting instead of being
+// produced one by one at the client's own pace.
 //
 // Differences from the reference, all inside this private contract:
 //  * queues are single-producer/single-consumer rings with acquire/release
@@ -74,14 +77,23 @@ struct Dim3 {
 
 // By-value copy of the arguments of one intercepted call (reference:
 // struct func_record, src/cuda_capture/intercept_temp.h:642-691).
+// Where the scheduler leaves the outcome of a record whose caller waits for it:
+// storage of the waiting call itself, not of the queue slot, which another
+// thread of the same client may be writing its next record into by the time
+// the waiter wakes up.
+struct WaitCell {
+  int32_t status;           // HIP status of the issued call, or kRecordGranted
+  hipStream_t sync_stream;  // granted calls: the stream the scheduler assigned
+};
+
 struct Record {
   int32_t type;
-  // Written by the scheduler before it retires the record; read by the caller
-  // after the hand-off completes.
+  // caller -> scheduler: 0, kRecordIssued or kRecordDeferred
   int32_t status;
-  // Set by the scheduler for synchronous copies: the stream the copy was
-  // enqueued on; the caller waits for it on its own thread.
-  hipStream_t sync_stream;
+  // Non-null when the caller waits for the record: written by the scheduler
+  // before it retires the record, read by the caller once the queue's head has
+  // passed the record's ticket.
+  WaitCell* cell;
   union {
     struct {
       const void* func;
@@ -136,6 +148,7 @@ struct Record {
 constexpr int32_t kRecordGranted = -1000;  // scheduler -> caller: run it yourself
 constexpr int32_t kRecordIssued = -1001;   // caller -> scheduler: already issued
 constexpr int32_t kRecordDeferred = -1002; // caller -> scheduler: nobody waits for the status
+constexpr int32_t kRecordPending = -1003;  // a WaitCell nobody has written yet
 
 constexpr int kMaxClients = 32;
 constexpr uint32_t kQueueSlots = 64;  // power of two; how far a best-effort client runs ahead
@@ -152,6 +165,10 @@ struct SlotAux {
   size_t kernarg_size;
   void* extra[5];
   hipGraphNode_t holder;
+  // the kernel `holder` was created for.  A node is only ever given new
+  // parameters for that same kernel; a launch of another kernel through this
+  // slot gets a fresh node.
+  const void* holder_func;
 };
 
 // The members are grouped by who writes them, one cache line (or more) per
@@ -176,6 +193,9 @@ struct alignas(64) ClientChannel {
   // postponed (see postpone_release)
   std::atomic<uint64_t> deferred_upto;
   std::atomic<int64_t> block_calls;     // highest it+1 the client passed to block()
+  // 1: this client's deferrable records may be queued without a waiting caller
+  // (set by orion_capture_allow_run_ahead after every arm; 0 after arm)
+  std::atomic<int> may_run_ahead;
 
   // -- written by the scheduler
   alignas(64) std::atomic<uint64_t> head;
@@ -207,10 +227,12 @@ struct alignas(64) ClientChannel {
 struct CaptureState {
   std::atomic<int> armed;        // 0 = pass everything through
   // 1 (ORION_BE_RUN_AHEAD=1): best-effort clients (every client but the last)
-  // queue deferrable records without waiting.  Off by default, and while a
-  // profile is captured (every kernel is timed where it is issued).
+  // that have been cleared for it (ClientChannel::may_run_ahead) queue
+  // deferrable records without waiting.  Off by default, and while a profile is
+  // captured (every kernel is timed where it is issued).
   std::atomic<int> run_ahead;
-  // 0 (ORION_BE_RUN_AHEAD_HOLDERS=0): hipLaunchKernel is never queued ahead
+  // 0: hipLaunchKernel is never queued ahead.  Only the host-only tests on the
+  // stand-in runtime can clear it (ORION_BE_RUN_AHEAD_HOLDERS=0 there).
   std::atomic<int> run_ahead_holders;
   std::atomic<uint32_t> epoch;   // bumped by every arm(): invalidates thread caches
   std::atomic<int> scheduler_polling;  // 1 while the scheduler thread is inside schedule()
@@ -228,6 +250,10 @@ extern "C" {
 orion::CaptureState* orion_capture_state(void);
 // Starts routing the given client threads through their queues.
 void orion_capture_arm(int num_clients, const int* client_tids, int scheduler_tid);
+// Clears (or bars) client `client` for queueing records ahead of their dispatch
+// under ORION_BE_RUN_AHEAD=1.  Every arm bars all clients again.  The scheduler
+// clears only clients whose work is made of this library's own kernels.
+void orion_capture_allow_run_ahead(int client, int allow);
 // Stops routing (everything passes through again) and wakes every waiter.
 void orion_capture_disarm(void);
 // Called by the scheduler thread right after it has set scheduler_polling on its

@@ -50,6 +50,13 @@ void resolve() {
       abort();
     }
   }
+  // the host-only stand-in is recognised by its own control call, not by how it
+  // was named: a real runtime named through the variable is still a real runtime
+  g_api.stand_in = dlsym(handle, "fakehip_set_costs") != nullptr;
+  // ORION_STAND_IN_AS_DEVICE=1: a host test asks to be treated like a GPU
+  // process (the variable can only take privileges away)
+  if (const char* strict = getenv("ORION_STAND_IN_AS_DEVICE"))
+    if (atoi(strict) != 0) g_api.stand_in = false;
   snprintf(chosen, sizeof chosen, "%s", from);
   g_api.library_path = chosen;
 #define X(name, ret, params) g_api.name = (decltype(g_api.name))dlsym(handle, #name);

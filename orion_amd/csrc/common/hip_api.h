@@ -127,6 +127,9 @@ struct HipApi {
   ORION_HIP_FUNCTIONS(X)
 #undef X
   const char* library_path;  // where the table came from
+  // True when the table came from the host-only stand-in runtime of the tests
+  // (recognised by its control entry point), which launches nothing on a GPU.
+  bool stand_in;
 };
 
 }  // namespace orion

@@ -224,9 +224,12 @@ int orion_profile_run(int until_iteration) {
     }
     Record* rec = &ch.slots[head & (kQueueSlots - 1)];
     ch.last_stream.store(run.stream, std::memory_order_release);
+    // the outcome goes to the waiting caller's own storage, before head moves
+    WaitCell* cell = rec->cell;
+    int status = (int)hipSuccess;
     if (orion_record_runs_on_caller(rec->type)) {
-      rec->sync_stream = run.stream;
-      rec->status = kGrantedToCaller;
+      if (cell) cell->sync_stream = run.stream;
+      status = kGrantedToCaller;
     } else if (rec_class_of(rec->type) == REC_KERNEL) {
       Row row;
       row.iteration = run.iteration;
@@ -235,11 +238,12 @@ int orion_profile_run(int until_iteration) {
       row.start = run.event();
       row.stop = run.event();
       row.ns = 0;
-      rec->status = launch_timed(*rec, run.stream, row.start, row.stop, hip);
+      status = launch_timed(*rec, run.stream, row.start, row.stop, hip);
       run.rows.push_back(std::move(row));
     } else {
-      rec->status = orion_execute_record(rec, run.stream);
+      status = orion_execute_record(rec, run.stream);
     }
+    if (cell) cell->status = status;
     ch.head.store(head + 1, std::memory_order_release);
   }
   orion_capture_state()->scheduler_polling.store(0, std::memory_order_release);

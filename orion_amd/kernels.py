@@ -55,10 +55,17 @@ def cu_masked_stream(cu_count, device=0):
 
 
 def _profiler_attached():
-    """True when a rocprofiler tool library is mapped into this process."""
+    """True when a rocprofiler *tool* library is in this process: rocprofv3
+    names it in ROCP_TOOL_LIBRARIES and LD_PRELOAD and it shows in the process's
+    maps.  (``librocprofiler-register.so`` does not count: the HIP runtime maps
+    it in every process, profiled or not.)"""
+    import os
+    named = os.environ.get("ROCP_TOOL_LIBRARIES", "") + ":" + os.environ.get("LD_PRELOAD", "")
+    if "rocprofiler-sdk-tool" in named:
+        return True
     try:
         with open("/proc/self/maps") as f:
-            return any("rocprofiler-sdk-tool" in line or "librocprofiler" in line for line in f)
+            return any("rocprofiler-sdk-tool" in line for line in f)
     except OSError:
         return False
 

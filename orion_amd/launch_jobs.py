@@ -72,15 +72,14 @@ def job_lists(config_dict_list):
                          "it selects the convolution solvers of the whole process")
     # ORION_BE_RUN_AHEAD=1 (best-effort clients queue their launches ahead of the
     # dispatch) has faulted an MI355X with framework trainers as best-effort
-    # clients, cause not found: refused for them unless explicitly overridden
+    # clients, cause not found: refused for them, with no override.  (The
+    # scheduler library never clears such a client for it either.)
     framework_be = [c for c in config_dict_list[:-1] if c in takes_flag]
-    if (os.environ.get("ORION_BE_RUN_AHEAD", "0") not in ("", "0") and framework_be
-            and os.environ.get("ORION_BE_RUN_AHEAD_UNSAFE", "0") in ("", "0")):
+    if os.environ.get("ORION_BE_RUN_AHEAD", "0") not in ("", "0") and framework_be:
         raise RuntimeError(
             "ORION_BE_RUN_AHEAD=1 with a framework model as a best-effort client has ended in "
             "GPU faults on an MI355X (ResNet-50 training beside ResNet-50 inference); it is "
-            "supported for the kernel-pair clients only.  Unset it, or set "
-            "ORION_BE_RUN_AHEAD_UNSAFE=1 to run anyway.")
+            "supported for the kernel-pair clients (gemm_bf16, triad_f32) only.  Unset it.")
     return {
         "model_names": [c["arch"] for c in config_dict_list],
         "model_files": [c["kernel_file"] for c in config_dict_list],

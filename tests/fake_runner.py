@@ -82,6 +82,10 @@ if os.environ.get("FAKE_RUNNER_MISCOUNT"):
     # submits per iteration
     records_per_iter[0] += int(os.environ["FAKE_RUNNER_MISCOUNT"])
 iters = [10_000] * n_be + [hp_iters]
+# FAKE_RUNNER_MODEL_NAMES=a,b,c: the model names setup() is given, one per client
+model_names = (os.environ["FAKE_RUNNER_MODEL_NAMES"].split(",")
+               if os.environ.get("FAKE_RUNNER_MODEL_NAMES") else ["fake"] * n_clients)
+assert len(model_names) == n_clients
 
 
 def write_profile(path, nk, seed):
@@ -276,7 +280,7 @@ def run_sched_untyped():
     handle_seen.append(handle)
     IntAr, CharAr, BoolAr = ctypes.c_int * n, ctypes.c_char_p * n, ctypes.c_bool * n
     tids_ar, nk_ar, ni_ar = IntAr(*tids), IntAr(*records_per_iter), IntAr(*iters)
-    names_ar = CharAr(*[b"fake"] * n)
+    names_ar = CharAr(*[m.encode() for m in model_names])
     files_ar = CharAr(*[f.encode("utf-8") for f in files])
     train = [True] * n_be + [False]
     train_ar = BoolAr(*train)
@@ -301,7 +305,7 @@ def run_sched():
     if untyped:
         return run_sched_untyped()
     sched_tid.append(threading.get_native_id())
-    py.run_scheduler(barriers, tids, ["fake"] * n_clients, files,
+    py.run_scheduler(barriers, tids, model_names, files,
                      [None] * n_clients, records_per_iter, [None] * n_clients,
                      iters, True, True, algo == "reef", algo == "sequential",
                      8 if algo == "reef" else 100_000, 1, 1, [True] * n_be + [False])

@@ -353,26 +353,44 @@ struct FakeKernelNode {
   void* slots[4];
   unsigned char storage[4][8];
 };
-// `bounds_of`: the kernel whose launch bounds the new block is checked against.
-// The runtime this stands in for checks a node's new parameters against the
-// kernel the node *holds* (hipGraphKernelNodeSetParams on a node whose kernel
-// has smaller bounds than the new block fails with hipErrorLaunchFailure).
+// `held`: the kernel the node holds when the call arrives (for a new node, the
+// kernel it is being created for).  This stand-in is the pessimistic reading of
+// what has been observed of the real runtime, which checks a node's new
+// parameters against the launch bounds of the kernel the node *holds*
+// (hipGraphKernelNodeSetParams on a node whose kernel has smaller bounds than
+// the new block fails with hipErrorLaunchFailure): here the argument copy, too,
+// follows the held kernel's argument list -- its count and sizes -- so a node
+// that is given another kernel's parameters ends up with truncated or missing
+// arguments, and a library that re-points nodes computes wrong results on the
+// host.  Such calls are counted (fakehip_repointed_nodes).
+std::atomic<long> g_repointed{0};
 static hipError_t fake_node_set(FakeKernelNode* n, const hipKernelNodeParams* p,
-                                const void* bounds_of) {
-  size_t sizes[4];
+                                const void* held) {
+  size_t sizes[4], held_sizes[4];
   const int count = fake_signature(p->func, sizes);
   if (count < 0 || p->kernelParams == nullptr) return hipErrorInvalidDeviceFunction;
-  if (p->blockDim.x * p->blockDim.y * p->blockDim.z > fake_launch_bounds(bounds_of))
+  if (p->blockDim.x * p->blockDim.y * p->blockDim.z > fake_launch_bounds(held))
     return hipErrorLaunchFailure;
+  int copy_count = count;
+  const size_t* copy_sizes = sizes;
+  if (held != p->func) {
+    g_repointed.fetch_add(1);
+    copy_count = fake_signature(held, held_sizes);
+    if (copy_count > count) copy_count = count;   // reads no further than the list given
+    copy_sizes = held_sizes;
+  }
   n->params = *p;
-  for (int i = 0; i < count; ++i) {
-    memcpy(n->storage[i], p->kernelParams[i], sizes[i]);
-    n->slots[i] = n->storage[i];
+  memset(n->storage, 0, sizeof n->storage);
+  for (int i = 0; i < count; ++i) n->slots[i] = n->storage[i];
+  for (int i = 0; i < copy_count; ++i) {
+    const size_t bytes = copy_sizes[i] < sizes[i] ? copy_sizes[i] : sizes[i];
+    memcpy(n->storage[i], p->kernelParams[i], bytes);
   }
   n->params.kernelParams = n->slots;
   n->params.extra = nullptr;
   return hipSuccess;
 }
+long fakehip_repointed_nodes(void) { return g_repointed.load(); }
 hipError_t hipGraphCreate(hipGraph_t* g, unsigned int) {
   *g = (hipGraph_t) new FakeGraph{0};
   return hipSuccess;

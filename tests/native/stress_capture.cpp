@@ -24,6 +24,7 @@
 extern "C" void fake_kernel_saxpy(void** p);
 extern "C" void fake_kernel_sqadd(void** p);
 extern "C" void fakehip_set_costs(long long kernel_ns, long long copy_ns);
+extern "C" long fakehip_repointed_nodes(void);
 extern "C" void orion_register_stream(void* stream);
 
 namespace {
@@ -227,7 +228,26 @@ void client(int c) {
         std::lock_guard<std::mutex> hold(g_worker_lock);
         g_worker_tasks.push_back({&st, half, nk, it, &done});
       }
-      while (!done.load(std::memory_order_acquire)) usleep(5);
+      // Meanwhile this thread makes blocking calls of its own: two threads of
+      // one client in the queue at once, one waiting for each of its records,
+      // the other (when records are queued ahead) racing up to a whole ring
+      // ahead of it.  Each blocking call must be carried out and must hand back
+      // its own result: x does not change during an iteration.
+      long reads = 0;
+      while (!done.load(std::memory_order_acquire)) {
+        float got[kN];
+        memset(got, 0xee, sizeof got);
+        if (hipMemcpy(got, st.x, kN * 4, hipMemcpyDeviceToHost) != hipSuccess) exit(10);
+        if (memcmp(got, st.host_x, sizeof got) != 0) {
+          fprintf(stderr, "client %d: a blocking copy made while another thread of the client "
+                          "launches was not carried out (iteration %d, read %ld)\n", c, it, reads);
+          exit(11);
+        }
+        float* scratch = nullptr;
+        if (hipMalloc((void**)&scratch, 256) != hipSuccess || scratch == nullptr) exit(12);
+        if (hipFree(scratch) != hipSuccess) exit(12);
+        ++reads;
+      }
     }
     if (it % 3 == 2) check_now(st, it, ev);
     block(it);
@@ -309,6 +329,10 @@ int main(int argc, char** argv) {
   }
   printf("%ld pooled blocks returned to the runtime while the clients ran\n", g_trimmed.load());
   if (g_trimmed.load() == 0) bad = 1;
+  // no graph kernel node may ever be given the parameters of another kernel
+  // than the one it was created for
+  printf("%ld graph kernel nodes re-pointed to another kernel\n", fakehip_repointed_nodes());
+  if (fakehip_repointed_nodes() != 0) bad = 1;
   if (g_done.back() != hp_iters) bad = 1;
   return bad;
 }

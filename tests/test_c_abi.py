@@ -94,3 +94,17 @@ def test_control_calls_are_noops_when_not_armed():
     cap.block(0)               # returns at once: nothing is armed
     assert cap.stop() == 0
     assert cap.orion_client_index() == -1
+
+
+def test_profiler_detection_counts_the_tool_library_only(monkeypatch):
+    """The kernel library is unloaded at exit only under a profiler.  The HIP
+    runtime maps librocprofiler-register.so in every process, so that library
+    must not count as one (it did: the kernel library was then unloaded at the
+    end of every run and never showed among the process's libraries)."""
+    import torch  # noqa: F401  (maps the HIP runtime and what it depends on)
+    from orion_amd import kernels
+    monkeypatch.delenv("ROCP_TOOL_LIBRARIES", raising=False)
+    monkeypatch.delenv("LD_PRELOAD", raising=False)
+    assert not kernels._profiler_attached()
+    monkeypatch.setenv("ROCP_TOOL_LIBRARIES", "/opt/rocm/lib/rocprofiler-sdk/librocprofiler-sdk-tool.so")
+    assert kernels._profiler_attached()

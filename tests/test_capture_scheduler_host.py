@@ -34,7 +34,7 @@ FAKEHIP = os.path.join(ROOT, "tests", "fakehip", "libfakehip.so")
 
 
 def run_child(workdir, algo, n_be, hp_iters, direct=True, graph=False, pin=True,
-              untyped=False, run_ahead=True, async_exec=False):
+              untyped=False, run_ahead=True, async_exec=False, extra_env=None):
     if not os.path.exists(FAKEHIP):
         pytest.fail("tests/fakehip/libfakehip.so is not built (make -C orion_amd/csrc)")
     proc = subprocess.run(
@@ -47,7 +47,7 @@ def run_child(workdir, algo, n_be, hp_iters, direct=True, graph=False, pin=True,
                  ORION_BE_RUN_AHEAD="1" if run_ahead else "0",
                  # the stand-in runtime runs queued work later, stream by stream in
                  # an order of its own choosing, instead of at the call
-                 FAKEHIP_ASYNC="1" if async_exec else "0"))
+                 FAKEHIP_ASYNC="1" if async_exec else "0", **(extra_env or {})))
     assert proc.returncode == 0, proc.stdout + proc.stderr
     line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
     return json.loads(line)
@@ -129,6 +129,29 @@ def test_every_record_is_handed_over_synchronously_by_default(tmp_path):
     obs = open(os.path.join(str(tmp_path), "observations.log")).read()
     dec = open(os.path.join(str(tmp_path), "decisions.log")).read()
     assert obslog.replay(obs) == dec and jobs.native_replay(obs) == dec
+
+
+def test_only_clients_of_the_librarys_own_kernels_queue_ahead(tmp_path):
+    """ORION_BE_RUN_AHEAD=1 in a GPU process: setup() clears a best-effort client
+    for queueing ahead by its model name -- the two hand-written kernel clients
+    only.  A framework model keeps the synchronous hand-off whatever the
+    environment says (with a trainer queueing ahead a GPU has faulted, cause not
+    found), and no variable overrides that.  The stand-in runtime asks to be
+    treated like a device here; by itself it clears every client, which is what
+    the other host tests rely on."""
+    strict = {"ORION_STAND_IN_AS_DEVICE": "1", "ORION_BE_RUN_AHEAD_UNSAFE": "1",
+              "FAKE_RUNNER_MODEL_NAMES": "resnet50,triad_f32,gemm_bf16"}
+    res = run_child(str(tmp_path), "orion", 2, 30, extra_env=strict)
+    assert not any(res["alive"]) and all(res["outputs_equal"]), res
+    assert res["deferred"][0] == 0 and res["deferred"][2] == 0
+    assert 0 < res["deferred"][1] < res["submitted"][1]
+    obs = open(os.path.join(str(tmp_path), "observations.log")).read()
+    dec = open(os.path.join(str(tmp_path), "decisions.log")).read()
+    assert obslog.replay(obs) == dec and jobs.native_replay(obs) == dec
+    # the knob that takes the graph kernel nodes out is for the stand-in only
+    strict["ORION_BE_RUN_AHEAD_HOLDERS"] = "0"
+    res = run_child(str(tmp_path), "orion", 2, 30, extra_env=strict)
+    assert res["holder_sets"] > 0, "ORION_BE_RUN_AHEAD_HOLDERS was honoured in a device process"
 
 
 @pytest.mark.parametrize("algo,n_be", [("orion", 1), ("orion", 2), ("reef", 1)])

@@ -256,14 +256,15 @@ def test_queueing_ahead_is_refused_for_framework_trainers(monkeypatch):
 
     trainer_pair = [entry("resnet50", True), entry("resnet50", False)]
     kernel_pair = [entry("triad_f32", True), entry("gemm_bf16", False)]
-    monkeypatch.delenv("ORION_BE_RUN_AHEAD_UNSAFE", raising=False)
     monkeypatch.setenv("ORION_BE_RUN_AHEAD", "0")
     lj.job_lists(trainer_pair)
     monkeypatch.setenv("ORION_BE_RUN_AHEAD", "1")
     lj.job_lists(kernel_pair)
     lj.job_lists([entry("triad_f32", True), entry("resnet50", False)])   # the model is the HP client
     lj.job_lists([entry("resnet50", False)])                              # a client alone
-    with pytest.raises(RuntimeError, match="kernel-pair clients only"):
+    with pytest.raises(RuntimeError, match="gemm_bf16, triad_f32"):
         lj.job_lists(trainer_pair)
+    # no environment variable opens the door again
     monkeypatch.setenv("ORION_BE_RUN_AHEAD_UNSAFE", "1")
-    lj.job_lists(trainer_pair)
+    with pytest.raises(RuntimeError, match="gemm_bf16, triad_f32"):
+        lj.job_lists(trainer_pair)
