@@ -130,6 +130,15 @@ void orion_thread_passthrough(int on);
 unsigned long long orion_client_submitted(int client);
 unsigned long long orion_client_deferred(int client);
 
+/* No reference counterpart: with ORION_CALL_TIMING=1 in the environment, the
+ * time the calling thread has spent so far inside the interposed kernel-launch
+ * and hipMemcpyAsync entry points (from entry to return, the runtime's own
+ * call included) and the number of such calls; both zero otherwise.  A client
+ * loop uses the pair to split a request's submission time into time inside the
+ * runtime and this library and time inside the framework. */
+unsigned long long orion_thread_time_in_calls_ns(void);
+unsigned long long orion_thread_calls(void);
+
 #ifdef __cplusplus
 }
 #endif

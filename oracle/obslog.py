@@ -15,10 +15,13 @@ Both logs are line-based text, shared with the native core
 (orion_amd/csrc/policy/obslog.h):
 
 observation log
-    ``J <n> <max_sms> <place_masks comma list> [L1] [R1]``  job header (L1: long
+    ``J <n> <max_sms> <place_masks comma list> [L1] [R1] [O1]``  job header (L1: long
                                                     best-effort kernels confined; R1:
                                                     the high-priority op's CU need
-                                                    is reserved)
+                                                    is reserved; O1: short kernels of
+                                                    the other class whose CU need
+                                                    exceeds the device go in alone,
+                                                    on the smallest mask)
     ``K <client> <num_kernels> <num_iters> <train 0|1> <profile path>``
     ``X <client> <num_kernels> <profile path>``      setup_change
     ``S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>``
@@ -101,10 +104,12 @@ class RecordingEnv(po.Env):
         self._dec = []
 
     # structure markers -------------------------------------------------
-    def header(self, max_sms, clients, confine_long=False, reserve_hp=False):
+    def header(self, max_sms, clients, confine_long=False, reserve_hp=False,
+               admit_oversized=False):
         self.confine_long = bool(confine_long)
         self.obs.append(f"J {self.n} {max_sms} " + ",".join(map(str, self.masks))
-                        + (" L1" if confine_long else "") + (" R1" if reserve_hp else ""))
+                        + (" L1" if confine_long else "") + (" R1" if reserve_hp else "")
+                        + (" O1" if admit_oversized else ""))
         for i, (nk, ni, train, path) in enumerate(clients):
             self.obs.append(f"K {i} {nk} {ni} {int(bool(train))} {path}")
 
@@ -161,10 +166,12 @@ class RecordingEnv(po.Env):
         self._us.append(us)
         return us
 
-    def dispatch(self, client, owner, cls, op_index, event_slot):
+    def dispatch(self, client, owner, cls, op_index, event_slot, smallest_mask=False):
         if cls != po.KERNEL:
             cu_slot = -1
         elif owner == self.n - 1:      # the high-priority stream is unmasked
+            cu_slot = 0
+        elif smallest_mask:            # an oversized kernel let in alone (O1)
             cu_slot = 0
         else:
             op = self.ops_of(client, op_index)
@@ -236,7 +243,7 @@ class ReplayEnv(po.Env):
             raise ReplayDivergence(f"poll {self.at}: unlogged time read")
         return self._us.pop(0)
 
-    def dispatch(self, *a):
+    def dispatch(self, *a, **kw):
         pass
 
     def iteration_done(self, *a):
@@ -252,7 +259,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
     oracle = None
     rec = None
     n = max_sms = masks = None
-    confine_long = reserve_hp = False
+    confine_long = reserve_hp = admit_oversized = False
     clients = {}
     lines = obs_text.splitlines()
     i = 0
@@ -262,9 +269,10 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
         if tag == "J":
             n, max_sms = int(parts[1]), int(parts[2])
             masks = [int(x) for x in parts[3].split(",")]
-            _ensure(set(parts[4:]) <= {"L1", "R1"} and len(parts) <= 6,
-                    "J: 3 fields and optional L1 / R1")
+            _ensure(set(parts[4:]) <= {"L1", "R1", "O1"} and len(parts) <= 7,
+                    "J: 3 fields and optional L1 / R1 / O1")
             confine_long, reserve_hp = "L1" in parts[4:], "R1" in parts[4:]
+            admit_oversized = "O1" in parts[4:]
         elif tag == "K":
             clients[int(parts[1])] = (int(parts[2]), int(parts[3]),
                                       bool(int(parts[4])), " ".join(parts[5:]))
@@ -280,7 +288,8 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
                 oracle = po.PolicyOracle(
                     [load_profile(c[3]) for c in order], [c[0] for c in order],
                     [c[1] for c in order], [c[2] for c in order], max_sms,
-                    sequential_fix=sequential_fix, reserve_hp=reserve_hp)
+                    sequential_fix=sequential_fix, reserve_hp=reserve_hp,
+                    admit_oversized=admit_oversized)
             polls = []
             i += 1
             while lines[i] != "E":

@@ -157,7 +157,14 @@ class PolicyOracle:
     ``schedule`` calls: seen, event_ids, cur_iters, penalty, profiles."""
 
     def __init__(self, profiles, num_kernels, num_iters, is_train, max_sms=80,
-                 sequential_fix=False, reserve_hp=False):
+                 sequential_fix=False, reserve_hp=False, admit_oversized=False):
+        # admit_oversized (not in the reference, whose CU clause :339-340 can
+        # never admit a kernel whose un-clipped need exceeds max_sms while a
+        # high-priority inference request is in flight): such a kernel goes in
+        # if nothing else has been admitted in this poll, its class and the
+        # running high-priority op's are both known and differ, and its
+        # duration is at most depth // 4; it is placed on the smallest mask.
+        self.admit_oversized = bool(admit_oversized)
         # reserve_hp (not in the reference): best-effort kernels admitted in one
         # poll may add up to max_sms minus the CU need of the high-priority op
         # last dispatched, instead of max_sms (:339 ignores that need).
@@ -193,11 +200,15 @@ class PolicyOracle:
         self.num_kernels[client] = int(num_kernels)
 
     # -- schedule_kernel + pop_from_queue (utils_sched.cpp:239-522, :113-117)
-    def _dispatch(self, env, client, owner, cls):
+    def _dispatch(self, env, client, owner, cls, smallest_mask=False):
         op_index = self.seen[client]
         # the event handed to schedule_kernel is events[owner][event_ids[owner]]
         # evaluated before the call, i.e. before the increment below
-        env.dispatch(client, owner, cls, op_index, self.event_ids[owner])
+        if smallest_mask:       # admit_oversized only: placement is forced
+            env.dispatch(client, owner, cls, op_index, self.event_ids[owner],
+                         smallest_mask=True)
+        else:
+            env.dispatch(client, owner, cls, op_index, self.event_ids[owner])
         if cls == KERNEL:            # every kernel-like case: :246-247 etc.
             self.event_ids[owner] += 1
             self.seen[client] += 1
@@ -334,6 +345,7 @@ class PolicyOracle:
                     cls = heads[j]
                     mem_op = cls in MEM_CLASSES
                     go = False
+                    oversized = False
                     if n == 1 or self.seen[hp] == 0 or mem_op:          # :333
                         go = True
                     elif (self.cur_iters[j] <= 10
@@ -348,6 +360,14 @@ class PolicyOracle:
                           and (op0.profile == -1 or profiles[hp] == -1
                                or profiles[hp] != op0.profile)):        # :340
                         go = True
+                    elif (self.admit_oversized and not self.is_train[hp]
+                          and size + op0.sm_used > room and size == 0
+                          and op0.sm_used > self.max_sms
+                          and op0.profile != -1 and profiles[hp] != -1
+                          and profiles[hp] != op0.profile
+                          and float(op0.duration) <= float(np.float32(depth // 4))):
+                        go = True
+                        oversized = True
                     if go and large_found:                   # :342-359
                         clear = True
                         for k in range(n - 1):
@@ -370,7 +390,7 @@ class PolicyOracle:
                         if (total > depth
                                 and self.cur_iters[hp] < self.max_iters[hp]):
                             large_found = True               # :366-368
-                        self._dispatch(env, j, j, cls)
+                        self._dispatch(env, j, j, cls, oversized)
                         start = j                            # :374
 
             finished = 0                                     # :380

@@ -108,6 +108,11 @@ class Backend:
     def stop(self):
         return bool(self.lib.stop()) or UNSCHEDULED_STOP.is_set()
 
+    def time_in_calls_ns(self):
+        """Time this thread has spent inside the interposed launch and copy
+        entry points (0 unless ORION_CALL_TIMING=1)."""
+        return int(self.lib.orion_thread_time_in_calls_ns())
+
     def register_stream(self, stream):
         self.lib.orion_register_stream(stream.cuda_stream)
 
@@ -182,13 +187,16 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
             if time.time() < next_startup:
                 continue
             t_begin = time.time()
+            in_calls = backend.time_in_calls_ns() if stamps is not None else 0
             step(batch_idx)
             t_submitted = time.time()
+            in_calls = backend.time_in_calls_ns() - in_calls if stamps is not None else 0
             backend.block(batch_idx)
             t_done = time.time()
             timings.append(t_done - next_startup)
             if stamps is not None:
-                stamps.append((t_begin - next_startup, t_submitted - t_begin, t_done - t_submitted))
+                stamps.append((t_begin - next_startup, t_submitted - t_begin,
+                               t_done - t_submitted, in_calls * 1e-9))
             if batch_idx >= WARMUP_ITERS and sleep_times[batch_idx] > 0:
                 next_startup += sleep_times[batch_idx]
             else:
@@ -218,7 +226,10 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
         # the percentiles only): lets runs be pooled
         data["latencies_ms"] = [round(float(t) * 1000, 4) for t in timings[drop:]]
         if stamps is not None:
-            for k, name in enumerate(("start_delay_ms", "submit_ms", "wait_ms")):
+            # submit_in_calls_ms: the part of submit_ms spent inside the interposed
+            # launch and copy calls (ORION_CALL_TIMING=1 and the library preloaded)
+            for k, name in enumerate(("start_delay_ms", "submit_ms", "wait_ms",
+                                      "submit_in_calls_ms")):
                 data[name] = [round(float(s[k]) * 1000, 4) for s in stamps[drop:]]
     write_result(tid, data)
     return data

@@ -39,6 +39,36 @@ thread_local int tl_client = kUncached;
 // the nested real call is not captured again.
 thread_local int tl_bypass = 0;
 
+// ORION_CALL_TIMING=1: every thread adds up the time it spends inside the
+// interposed launch and copy entry points (entry to return, the real call
+// included), for orion_thread_time_in_calls_ns: lets a client loop split a
+// request's submission time into "inside the runtime and this library" and
+// "inside the framework".  Off: one predictable branch per call.
+const bool g_call_timing = [] {
+  const char* e = getenv("ORION_CALL_TIMING");
+  return e && atoi(e) != 0;
+}();
+thread_local uint64_t tl_call_ns = 0;
+thread_local uint64_t tl_call_count = 0;
+thread_local int tl_call_depth = 0;
+
+struct CallTimer {
+  timespec t0;
+  bool on;
+  CallTimer() : on(g_call_timing && tl_call_depth++ == 0) {
+    if (on) clock_gettime(CLOCK_MONOTONIC, &t0);
+  }
+  ~CallTimer() {
+    if (!g_call_timing) return;
+    --tl_call_depth;
+    if (!on) return;
+    timespec t1;
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    tl_call_ns += (uint64_t)((t1.tv_sec - t0.tv_sec) * 1000000000ll + (t1.tv_nsec - t0.tv_nsec));
+    ++tl_call_count;
+  }
+};
+
 void flush_channel(ClientChannel& ch);   // defined with submit()
 void run_postponed(bool everything);     // likewise
 void postponed_fence();
@@ -59,20 +89,35 @@ inline void cpu_relax(unsigned& spins) {
 // kernel, as does a CPU set too small for one CPU per slot.
 struct Pinning {
   bool on = false;
+  bool clients = true;        // false: only the scheduler thread is pinned
+  int scheduler_slot = 0;
   int cpus[kMaxClients + 2];
   pid_t tid[kMaxClients + 1];
   cpu_set_t before[kMaxClients + 1];
 };
 Pinning g_pin;
 
+// ORION_PIN_THREADS: 1 every client thread and the scheduler thread (default),
+// 0 none, "scheduler" the scheduler thread only, "top" all of them but counted
+// down from the highest CPU the process may use instead of up from the second.
 void pinning_reset(int slots) {
   for (pid_t& t : g_pin.tid) t = 0;
   const char* env = getenv("ORION_PIN_THREADS");
   g_pin.on = false;
-  if (env && atoi(env) == 0) return;
+  g_pin.clients = !(env && strcmp(env, "scheduler") == 0);
+  g_pin.scheduler_slot = slots - 1;
+  const bool from_top = env && strcmp(env, "top") == 0;
+  if (env && strcmp(env, "0") == 0) return;
   cpu_set_t allowed;
   if (sched_getaffinity(getpid(), sizeof allowed, &allowed) != 0) return;
   int n = 0;
+  if (from_top) {
+    // slot s -> cpus[s + 1]; one more CPU must remain for everybody else
+    for (int c = CPU_SETSIZE - 1; c >= 0 && n < slots; --c)
+      if (CPU_ISSET(c, &allowed)) g_pin.cpus[1 + n++] = c;
+    g_pin.on = n == slots && CPU_COUNT(&allowed) > slots;
+    return;
+  }
   for (int c = 0; c < CPU_SETSIZE && n < slots + 1; ++c)
     if (CPU_ISSET(c, &allowed)) g_pin.cpus[n++] = c;
   g_pin.on = n == slots + 1;
@@ -80,6 +125,7 @@ void pinning_reset(int slots) {
 
 void pin_caller(int slot, pid_t tid) {
   if (!g_pin.on || g_pin.tid[slot] == tid) return;
+  if (!g_pin.clients && slot != g_pin.scheduler_slot) return;
   if (sched_getaffinity(0, sizeof(cpu_set_t), &g_pin.before[slot]) != 0) return;
   cpu_set_t one;
   CPU_ZERO(&one);
@@ -398,6 +444,12 @@ unsigned long long orion_client_deferred(int client) {
   if (client < 0 || client >= kMaxClients) return 0;
   return g_state.channels[client].deferred.load(std::memory_order_relaxed);
 }
+
+// Time the calling thread has spent inside the interposed launch and copy entry
+// points so far, and how many such calls it made (ORION_CALL_TIMING=1; zero
+// otherwise).
+unsigned long long orion_thread_time_in_calls_ns(void) { return tl_call_ns; }
+unsigned long long orion_thread_calls(void) { return tl_call_count; }
 
 // The client a call naming `stream` from the calling thread would be queued
 // for, or a negative value when it would go straight to the runtime.
@@ -782,8 +834,9 @@ int submit(int idx, Record& r, bool wait) {
     // The scheduler lets this client issue its own calls: run the call here, on
     // the stream the scheduler named, under the producer lock so that the
     // notices reach the queue in issue order; nobody waits for the notice.  The
-    // notice is the record's type alone: the scheduler reads nothing else of a
-    // call that has been made.
+    // notice is the record's type and, for a kernel, what was launched (kept for
+    // the scheduler's reports): the scheduler reads nothing else of a call that
+    // has been made.
     int st;
     if (orion_record_runs_on_caller(r.type)) {
       st = execute_on_caller(r, direct);
@@ -797,6 +850,7 @@ int submit(int idx, Record& r, bool wait) {
     slot->type = r.type;
     slot->status = kRecordIssued;
     slot->cell = nullptr;
+    slot->u.launch.func = record_function(r);   // which kernel: for the scheduler's reports
     ch.tail.store(ticket + 1, std::memory_order_release);
     ch.submitted.store(ch.submitted.load(std::memory_order_relaxed) + 1, std::memory_order_relaxed);
     ch.producer_lock.store(0, std::memory_order_release);
@@ -938,6 +992,7 @@ extern "C" {
 
 hipError_t hipLaunchKernel(const void* f, dim3 grid, dim3 block, void** args,
                            size_t shmem, hipStream_t stream) {
+  CallTimer timer;
   const int idx = client_for_call(stream);
   if (idx < 0) return orion_hip_api()->hipLaunchKernel(f, grid, block, args, shmem, stream);
   Record r;
@@ -975,6 +1030,7 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
                                  unsigned int gz, unsigned int bx, unsigned int by,
                                  unsigned int bz, unsigned int shmem,
                                  hipStream_t stream, void** params, void** extra) {
+  CallTimer timer;
   const int idx = client_for_call(stream);
   if (idx < 0)
     return orion_hip_api()->hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, shmem,
@@ -990,6 +1046,7 @@ hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t gx, uint32_t gy,
                                     uint32_t bz, size_t shmem, hipStream_t stream,
                                     void** params, void** extra, hipEvent_t start,
                                     hipEvent_t stop_ev, uint32_t flags) {
+  CallTimer timer;
   const int idx = client_for_call(stream);
   if (idx < 0)
     return orion_hip_api()->hipExtModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, shmem,
@@ -1114,6 +1171,7 @@ hipError_t hipMemcpy(void* dst, const void* src, size_t bytes, hipMemcpyKind kin
 
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes,
                           hipMemcpyKind kind, hipStream_t stream) {
+  CallTimer timer;
   const int idx = client_for_call(stream);
   if (idx < 0) return orion_hip_api()->hipMemcpyAsync(dst, src, bytes, kind, stream);
   Record r;

@@ -144,6 +144,20 @@ struct Record {
   } u;
 };
 
+// What a kernel-class record launches: the host function, the module function
+// or the executable graph.  Each is the first member of its struct, so a notice
+// of a call already made (which carries nothing else) stores it through
+// u.launch.func whatever the record's type.
+inline const void* record_function(const Record& r) {
+  if (r.type <= RT_COOP_LAUNCH_KERNEL) return r.u.launch.func;
+  if (r.type <= RT_MODULE_COOP_LAUNCH) return (const void*)r.u.module.f;
+  if (r.type == RT_GRAPH_LAUNCH) return (const void*)r.u.graph.exec;
+  return nullptr;
+}
+static_assert(offsetof(Record, u.launch.func) == offsetof(Record, u.module.f) &&
+              offsetof(Record, u.launch.func) == offsetof(Record, u.graph.exec),
+              "the launched object must be the first member of every kernel record");
+
 // Record::status values outside the HIP error range.
 constexpr int32_t kRecordGranted = -1000;  // scheduler -> caller: run it yourself
 constexpr int32_t kRecordIssued = -1001;   // caller -> scheduler: already issued

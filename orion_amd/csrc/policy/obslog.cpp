@@ -21,12 +21,13 @@ void appendf(std::string* s, const char* fmt, ...) {
 }  // namespace
 
 void Recorder::header(int max_sms, const std::vector<int>& masks, bool confine_long,
-                      bool reserve_hp) {
+                      bool reserve_hp, bool admit_oversized) {
   appendf(&obs_, "J %d %d ", n_, max_sms);
   for (size_t i = 0; i < masks.size(); ++i)
     appendf(&obs_, i ? ",%d" : "%d", masks[i]);
   if (confine_long) obs_ += " L1";  // long best-effort kernels are confined
   if (reserve_hp) obs_ += " R1";    // the high-priority op's CU need is reserved
+  if (admit_oversized) obs_ += " O1";  // oversized short kernels of the other class go in alone
   obs_ += '\n';
 }
 
@@ -233,7 +234,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
   };
 
   int n = 0, max_sms = 0;
-  bool confine_long = false, reserve_hp = false;
+  bool confine_long = false, reserve_hp = false, admit_oversized = false;
   std::vector<int> masks;
   std::vector<ClientDesc> clients;
   Policy* policy = nullptr;
@@ -248,14 +249,15 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
     const char tag = l[0];
     if (tag == 'J') {
       auto p = split(l, ' ', 7);
-      bool options_ok = p.size() >= 4 && p.size() <= 6;
+      bool options_ok = p.size() >= 4 && p.size() <= 7;
       for (size_t k = 4; options_ok && k < p.size(); ++k) {
         if (p[k] == "L1") confine_long = true;
         else if (p[k] == "R1") reserve_hp = true;
+        else if (p[k] == "O1") admit_oversized = true;
         else options_ok = false;
       }
       if (!options_ok) {
-        ok = bad(i, "J needs 3 fields and optional L1 / R1");
+        ok = bad(i, "J needs 3 fields and optional L1 / R1 / O1");
         break;
       }
       n = atoi(p[1].c_str());
@@ -305,7 +307,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
         }
         if (!ok) break;
         policy = new Policy(std::move(profs), nk, ni, tr, max_sms, masks,
-                            sequential_fix, confine_long, reserve_hp);
+                            sequential_fix, confine_long, reserve_hp, admit_oversized);
       }
       ScheduleArgs a;
       a.warmup = atoi(p[1].c_str()) != 0;

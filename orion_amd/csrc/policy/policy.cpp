@@ -135,7 +135,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
                std::vector<int> num_kernels, std::vector<int> num_iters,
                std::vector<bool> is_train, int max_sms,
                std::vector<int> cu_masks, bool sequential_fix, bool confine_long,
-               bool reserve_hp)
+               bool reserve_hp, bool admit_oversized)
     : n_((int)profiles.size()),
       ops_(std::move(profiles)),
       num_kernels_(std::move(num_kernels)),
@@ -146,6 +146,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
       sequential_fix_(sequential_fix),
       confine_long_(confine_long),
       reserve_hp_(reserve_hp),
+      admit_oversized_(admit_oversized),
       seen_(n_, 0),
       event_ids_(n_, 0),
       cur_iters_(n_, 0),
@@ -163,7 +164,8 @@ void Policy::setup_change(int client, std::vector<OpInfo> ops, int num_kernels) 
 
 // schedule_kernel + pop_from_queue: kernel-like records advance the client's
 // position in its profile and the owner's event index; memory records do not.
-void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class) {
+void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class,
+                      bool smallest_mask) {
   Dispatch d;
   d.client = client;
   d.owner = owner;
@@ -174,6 +176,8 @@ void Policy::dispatch(PolicyHost& host, int client, int owner, int rec_class) {
     d.cu_slot = -1;
   } else if (owner == n_ - 1) {
     d.cu_slot = 0;  // the high-priority stream spans the whole GPU
+  } else if (smallest_mask) {
+    d.cu_slot = 0;  // an oversized kernel let in beside a high-priority request
   } else {
     const OpInfo& op = ops_[client][d.op_index];
     d.cu_slot = place_cu_slot(cu_masks_, rec_class, op.sm_used, algo_,
@@ -336,6 +340,7 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
         const int cls = heads[j];
         const bool mem_op = is_mem_class(cls);
         bool go = false;
+        bool oversized = false;
         int outcome = ADM_REFUSED_CUS;
         if (n == 1 || seen_[hp] == 0 || mem_op) {
           go = true;
@@ -350,6 +355,12 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
           go = true;
         } else if (size + op0.sm_used <= room) {
           outcome = ADM_REFUSED_CLASS;
+        } else if (admit_oversized_ && !is_train_[hp] && size == 0 &&
+                   op0.sm_used > max_sms_ && op0.profile != -1 && profiles[hp] != -1 &&
+                   profiles[hp] != op0.profile &&
+                   op0.duration <= (float)(args.depth / 4)) {
+          go = true;
+          oversized = true;
         }
         if (go && large_found) {
           bool clear = true;
@@ -368,13 +379,13 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
             outcome = ADM_THROTTLED;
           }
         }
-        admission_[j][go ? ADM_ADMITTED : outcome] += 1;
+        admission_[j][go ? (oversized ? ADM_OVERSIZED : ADM_ADMITTED) : outcome] += 1;
         if (go) {
           size += op0.sm_used;
           if (!mem_op) sum = (long)((float)sum + op0.duration);
           if (sum > args.depth && cur_iters_[hp] < max_iters_[hp])
             large_found = true;
-          dispatch(host, j, j, cls);
+          dispatch(host, j, j, cls, oversized);
           start = j;
         }
       }

@@ -99,7 +99,9 @@ enum Admission : int {
   ADM_REFUSED_CLASS = 2,  // fits, but has the running high-priority op's class (:340)
   ADM_THROTTLED = 3,      // admissible, but the duration budget is spent and the
                           // best-effort streams have not drained (:342-359)
-  ADM_COUNT = 4
+  ADM_OVERSIZED = 4,      // admitted alone on the smallest mask although its CU
+                          // need exceeds the budget (option admit_oversized)
+  ADM_COUNT = 5
 };
 
 struct ScheduleArgs {
@@ -121,7 +123,8 @@ class Policy {
          std::vector<int> num_kernels, std::vector<int> num_iters,
          std::vector<bool> is_train, int max_sms,
          std::vector<int> cu_masks, bool sequential_fix,
-         bool confine_long = false, bool reserve_hp = false);
+         bool confine_long = false, bool reserve_hp = false,
+         bool admit_oversized = false);
 
   void setup_change(int client, std::vector<OpInfo> ops, int num_kernels);
 
@@ -141,7 +144,8 @@ class Policy {
   long sum() const { return sum_; }
 
  private:
-  void dispatch(PolicyHost& host, int client, int owner, int rec_class);
+  void dispatch(PolicyHost& host, int client, int owner, int rec_class,
+                bool smallest_mask = false);
   void reef(PolicyHost& host, const std::vector<int>& heads, int depth);
   int sequential(PolicyHost& host, const std::vector<int>& heads, int start);
 
@@ -164,6 +168,20 @@ class Policy {
   // op last dispatched.  A whole-GPU op -- a HIP-graph request -- then leaves
   // no room; short kernels with a small need leave nearly all of it.
   bool reserve_hp_;
+  // Admission option (not in the reference).  The reference's CU clause
+  // (size + sm_used <= max_sms, scheduler_eval.cpp:339-340) is written for a GPU
+  // without compute-unit masks, where a kernel's profiled need is what it will
+  // occupy; the need is not clipped to the device, so a kernel whose grid alone
+  // exceeds the device can never be admitted while a high-priority inference
+  // request is in flight and its whole client stands behind it.  On a CU-masked
+  // stream the kernel occupies the mask, whatever its grid.  With the option
+  // such a kernel is admitted while a request is in flight if it is the first
+  // best-effort kernel admitted in the poll (size == 0: it is let in alone, and
+  // its full need then closes the poll's budget), its class and the class of
+  // the running high-priority op are both known and differ, and its profiled
+  // duration is at most a quarter of the duration budget; it goes to the
+  // smallest mask.  Everything else is the reference's rule.
+  bool admit_oversized_;
   // survive between schedule() calls, like the reference's globals
   std::vector<int> seen_;
   std::vector<int> event_ids_;

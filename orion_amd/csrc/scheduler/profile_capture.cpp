@@ -9,7 +9,6 @@
 // Reference counterpart: the offline Nsight Compute / Nsight Systems runs of
 // PROFILE.md:7-54 and profiling/postprocessing/process_ncu.py; there the row
 // count has to be matched by hand against what the interposers capture.
-#include <cxxabi.h>
 #include <immintrin.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -21,6 +20,7 @@
 #include <vector>
 
 #include "../capture/capture.h"
+#include "../common/kernel_name.h"
 
 extern "C" {
 int orion_execute_record(const orion::Record* rec, hipStream_t stream);
@@ -43,21 +43,7 @@ struct Row {
   float ns;
 };
 
-std::string short_name(const char* mangled) {
-  if (!mangled || !*mangled) return "unknown";
-  int status = 0;
-  char* dem = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
-  std::string s = (status == 0 && dem) ? dem : mangled;
-  free(dem);
-  // cut template and call arguments; the profile CSV is split on ','
-  for (size_t at; (at = s.find("(anonymous namespace)::")) != std::string::npos;)
-    s.erase(at, strlen("(anonymous namespace)::"));
-  size_t cut = s.find_first_of("<(");
-  if (cut != std::string::npos && cut > 0) s = s.substr(0, cut);
-  for (char& c : s)
-    if (c == ',' || c == '\n') c = ';';
-  return s;
-}
+std::string short_name(const char* mangled) { return short_kernel_name(mangled); }
 
 struct CaptureRun {
   const HipApi* hip = nullptr;

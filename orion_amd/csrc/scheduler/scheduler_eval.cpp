@@ -38,6 +38,7 @@
 #include <vector>
 
 #include "../capture/capture.h"
+#include "../common/kernel_name.h"
 #include "../policy/obslog.h"
 #include "../policy/policy.h"
 #include "orion_scheduler.h"
@@ -95,6 +96,8 @@ class LiveHost : public PolicyHost {
     last_slot_.assign((size_t)n, -1);
     last_kernel_stream_.assign((size_t)n, nullptr);
     client_stream_.assign((size_t)n, nullptr);
+    used_streams_.resize((size_t)n);
+    live_rows_.resize((size_t)n);
     cur_cu_slot_.assign((size_t)n, -1);
     start_pending_.assign((size_t)n, true);
     iter_start_.assign((size_t)n, Clock::now());
@@ -146,10 +149,19 @@ class LiveHost : public PolicyHost {
   void set_policy(const Policy* p) { policy_ = p; }
 
   // ---- PolicyHost
+  // One pause per poll while things happen; after a run of polls that changed
+  // nothing (no record anywhere, or everything waiting for the GPU) a few more:
+  // the loop then leaves the core's shared execution resources, and the
+  // runtime's locks behind hipEventQuery, to the client threads, at the price of
+  // a fraction of a microsecond before the next record is seen.
   void begin_poll() override {
     _mm_pause();
+    if (idle_polls_ > 32)
+      for (int i = 1; i < idle_pauses_; ++i) _mm_pause();
     if ((++polls_ & 0xfffff) == 0) watchdog();
   }
+
+  void end_poll(bool effective) override { idle_polls_ = effective ? 0 : idle_polls_ + 1; }
 
   bool stop_ack(int client) override {
     return cap_->channels[client].stop_ack.load(std::memory_order_acquire) != 0;
@@ -217,7 +229,8 @@ class LiveHost : public PolicyHost {
         die("client " + std::to_string(d.client) + " submits more kernel records per "
             "iteration than the " + std::to_string(policy_->num_kernels()[(size_t)d.client]) +
             " its profile names: " + std::to_string(done) + " iterations completed by count, "
-            "block() called " + std::to_string(blocked) + " times");
+            "block() called " + std::to_string(blocked) + " times" +
+            where_it_differs(d.client, rec));
     }
 
     // Stream: the owner's stream set, at the slot the policy placed the kernel
@@ -256,6 +269,10 @@ class LiveHost : public PolicyHost {
       // already (as every queued call of the reference does); if the real call
       // fails now there is nobody to tell, so the job ends here.
       const int status = orion_execute_record(rec, stream);
+      auto& used = used_streams_[(size_t)d.client];
+      bool known = false;
+      for (hipStream_t u : used) known = known || u == stream;
+      if (!known) used.push_back(stream);
       if (cell) {
         cell->status = status;
       } else if (status != (int)hipSuccess) {
@@ -267,6 +284,9 @@ class LiveHost : public PolicyHost {
       }
     }
     if (d.rec_class == REC_KERNEL) {
+      auto& rows = live_rows_[(size_t)d.client];
+      if (d.op_index == 0) rows.clear();
+      if ((size_t)d.op_index == rows.size()) rows.push_back({rec->type, record_function(*rec)});
       last_kernel_stream_[(size_t)d.owner] = stream;
       last_slot_[(size_t)d.owner] = d.event_slot;
       last_recorded_[(size_t)d.owner] = false;
@@ -283,12 +303,86 @@ class LiveHost : public PolicyHost {
 
   void iteration_done(int client, int iteration) override {
     ClientChannel& ch = cap_->channels[client];
+    // The policy has just seen the iteration's last kernel complete: every
+    // stream the client's records went to is idle, and this thread now waits
+    // for each of them once, which costs nothing on the GPU and lets the runtime
+    // release the commands it has kept for the stream.  Nobody else ever waits
+    // for these streams (a client's own waits are answered from here: block()),
+    // and the runtime, left alone, releases a stream's commands only when about
+    // a thousand have piled up -- in the middle of a later iteration, inside
+    // whichever launch hits the limit (measured on a ResNet-50 request of 371
+    // launches issued by the client itself: every 8th of 3 requests took 0.6 ms
+    // longer to submit, 35 us with an empty kernel).  Before the release, so
+    // that the client cannot yet be adding work to the stream being waited for.
+    for (hipStream_t s : used_streams_[(size_t)client]) (void)hip_->hipStreamSynchronize(s);
+    used_streams_[(size_t)client].clear();
+    if (hipStream_t direct = ch.direct_stream.load(std::memory_order_relaxed))
+      (void)hip_->hipStreamSynchronize(direct);
     ch.released_iters.store((int64_t)iteration + 1, std::memory_order_release);
     const float ms = (float)iteration_us(client) / 1000.0f;
     durations_ms_[(size_t)client].push_back(ms);
     start_pending_[(size_t)client] = true;
     last_progress_ = Clock::now();
     if (client == update_owner_) update_valid_ = false;
+  }
+
+  // Name of what a kernel-class record launches, as a profile's Name column
+  // would hold it.
+  std::string launched_name(int32_t type, const void* function) const {
+    if (type == RT_GRAPH_LAUNCH) return "hipGraphLaunch";
+    const char* raw = nullptr;
+    if (type <= RT_COOP_LAUNCH_KERNEL) {
+      if (hip_->hipKernelNameRefByPtr) raw = hip_->hipKernelNameRefByPtr(function, nullptr);
+    } else if (hip_->hipKernelNameRef) {
+      raw = hip_->hipKernelNameRef((hipFunction_t)function);
+    }
+    return short_kernel_name(raw);
+  }
+
+  // Where a client's iteration leaves its profile: the first row whose name
+  // differs from the kernel the client launched there, with both names -- which
+  // is what tells a changed convolution solver or an extra cast kernel apart
+  // from a wrong num_kernels.  `extra`: a kernel record beyond the profile's
+  // last row (the head of the client's queue), or null.
+  std::string where_it_differs(int client, const Record* extra = nullptr) const {
+    if (!policy_) return "";
+    const auto& ops = policy_->ops(client);
+    const auto& rows = live_rows_[(size_t)client];
+    const int nk = policy_->num_kernels()[(size_t)client];
+    char line[512];
+    for (size_t i = 0; i < rows.size() && i < ops.size(); ++i) {
+      const std::string live = launched_name(rows[i].type, rows[i].function);
+      if (live != ops[i].name) {
+        snprintf(line, sizeof line,
+                 "\n  client %d: first difference at profile row %zu: the profile names '%s', "
+                 "the client launched '%s'", client, i, ops[i].name.c_str(), live.c_str());
+        return line;
+      }
+    }
+    std::string out;
+    snprintf(line, sizeof line, "\n  client %d: the %zu kernels launched so far in this iteration "
+             "carry the names of profile rows 0..%zu", client, rows.size(),
+             rows.empty() ? 0 : rows.size() - 1);
+    out = rows.empty() ? "" : line;
+    if (extra && rec_class_of(extra->type) == REC_KERNEL) {
+      snprintf(line, sizeof line, "\n  client %d: after the profile's last row (%d rows) it "
+               "launched '%s'", client, nk,
+               launched_name(extra->type, record_function(*extra)).c_str());
+      out += line;
+    } else if ((int)rows.size() < nk && rows.size() < ops.size()) {
+      snprintf(line, sizeof line, "\n  client %d: the profile's next row (%zu of %d) names '%s'",
+               client, rows.size(), nk, ops[rows.size()].name.c_str());
+      out += line;
+    }
+    return out;
+  }
+
+  // The record at the head of a client's queue, or null.
+  const Record* head_record(int client) const {
+    ClientChannel& ch = cap_->channels[client];
+    const uint64_t head = ch.head.load(std::memory_order_relaxed);
+    if (ch.tail.load(std::memory_order_acquire) == head) return nullptr;
+    return &ch.slots[head & (kQueueSlots - 1)];
   }
 
   void set_stop(int client) override {
@@ -321,6 +415,7 @@ class LiveHost : public PolicyHost {
                policy_->seen()[(size_t)i], policy_->num_kernels()[(size_t)i], queued, blocked,
                released, policy_->cur_iters()[(size_t)i]);
       dump += line;
+      if (blocked > released || queued > 0) dump += where_it_differs(i);
     }
     if (!someone_waits) {
       last_progress_ = now;
@@ -368,6 +463,9 @@ class LiveHost : public PolicyHost {
   std::vector<int> masks_;
   const Policy* policy_ = nullptr;
   uint64_t polls_ = 0;
+  uint32_t idle_polls_ = 0;   // polls in a row that changed nothing
+  const int idle_pauses_ = getenv("ORION_IDLE_PAUSES") && atoi(getenv("ORION_IDLE_PAUSES")) > 0
+                               ? atoi(getenv("ORION_IDLE_PAUSES")) : 8;
   Clock::time_point last_progress_ = Clock::now();
   double stuck_limit_s_ = getenv("ORION_STUCK_LIMIT_S") ? atof(getenv("ORION_STUCK_LIMIT_S")) : 20.0;
   const HipApi* hip_;
@@ -377,6 +475,13 @@ class LiveHost : public PolicyHost {
   std::vector<char> last_recorded_;
   std::vector<int> last_slot_;
   std::vector<hipStream_t> last_kernel_stream_, client_stream_;
+  // streams this thread has issued records of the client's current iteration on
+  std::vector<std::vector<hipStream_t>> used_streams_;
+  // What the client launched at each profile row of its current iteration
+  // (record type and the launched function): resolved to names only when a
+  // count mismatch has to be reported.
+  struct LiveRow { int32_t type; const void* function; };
+  std::vector<std::vector<LiveRow>> live_rows_;
   std::vector<int> cur_cu_slot_;
   hipEvent_t update_event_ = nullptr;
   int update_owner_ = -1, update_slot_ = -1;
@@ -430,14 +535,18 @@ void write_admission_summary() {
     char line[256];
     snprintf(line, sizeof line,
              "%s{\"client\": %d, \"admitted\": %llu, \"refused_cu_budget\": %llu, "
-             "\"refused_same_class\": %llu, \"throttled\": %llu}", i ? ", " : "", i,
-             (unsigned long long)a[ADM_ADMITTED], (unsigned long long)a[ADM_REFUSED_CUS],
-             (unsigned long long)a[ADM_REFUSED_CLASS], (unsigned long long)a[ADM_THROTTLED]);
+             "\"refused_same_class\": %llu, \"throttled\": %llu, \"admitted_oversized\": %llu}",
+             i ? ", " : "", i,
+             (unsigned long long)(a[ADM_ADMITTED] + a[ADM_OVERSIZED]),
+             (unsigned long long)a[ADM_REFUSED_CUS], (unsigned long long)a[ADM_REFUSED_CLASS],
+             (unsigned long long)a[ADM_THROTTLED], (unsigned long long)a[ADM_OVERSIZED]);
     json += line;
     if (g.verbose && i < g.n - 1)
-      printf("Client %d: polls with a record waiting: %llu admitted, %llu over the CU budget, "
+      printf("Client %d: polls with a record waiting: %llu admitted (%llu of them oversized, "
+             "alone on the smallest mask), %llu over the CU budget, "
              "%llu same class as the high-priority op, %llu throttled by the duration budget\n",
-             i, (unsigned long long)a[ADM_ADMITTED], (unsigned long long)a[ADM_REFUSED_CUS],
+             i, (unsigned long long)(a[ADM_ADMITTED] + a[ADM_OVERSIZED]),
+             (unsigned long long)a[ADM_OVERSIZED], (unsigned long long)a[ADM_REFUSED_CUS],
              (unsigned long long)a[ADM_REFUSED_CLASS], (unsigned long long)a[ADM_THROTTLED]);
   }
   json += "]}\n";
@@ -511,8 +620,12 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** models,
   // Admission option: reserve the high-priority op's own CU need (see policy.h).
   const bool reserve_hp = getenv("ORION_RESERVE_HP_CUS") &&
                           atoi(getenv("ORION_RESERVE_HP_CUS")) != 0;
+  // Admission option: let short best-effort kernels of the opposite class whose
+  // CU need exceeds the device in alone, on the smallest mask (see policy.h).
+  const bool admit_oversized = getenv("ORION_ADMIT_OVERSIZED") &&
+                               atoi(getenv("ORION_ADMIT_OVERSIZED")) != 0;
   g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, max_sms, g.masks,
-                            !as_written, confine_long, reserve_hp));
+                            !as_written, confine_long, reserve_hp, admit_oversized));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
   g.host->set_policy(g.policy.get());
   g.recorder.reset();
@@ -521,7 +634,7 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** models,
     if (*dir) {
       g.record_dir = dir;
       g.recorder.reset(new Recorder(g.host.get(), num_clients));
-      g.recorder->header(max_sms, g.masks, confine_long, reserve_hp);
+      g.recorder->header(max_sms, g.masks, confine_long, reserve_hp, admit_oversized);
       for (int i = 0; i < num_clients; ++i)
         g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
       // start both logs afresh
@@ -610,7 +723,8 @@ void* schedule(void* /*scheduler*/, int num_clients, bool profile_mode, int /*it
       if (g.host->waiting_class(i) == REC_KERNEL)
         die("client " + std::to_string(i) + " submits more kernel records per iteration "
             "than the " + std::to_string(g.policy->num_kernels()[(size_t)i]) +
-            " its profile names: one is still queued after the iteration was released");
+            " its profile names: one is still queued after the iteration was released" +
+            g.host->where_it_differs(i, g.host->head_record(i)));
   }
   if (g.recorder) {
     g.recorder->end_schedule();

@@ -22,12 +22,16 @@ Class.  The reference places a kernel left or right of the roofline's knee by
 its arithmetic intensity (flops / DRAM bytes against 9.72 flop/byte,
 roofline_analysis.py:51-62), i.e. it asks which of the two roofs the kernel is
 closer to.  The same question is answered here from busy fractions, which one
-counter each gives: the fraction of the kernel's time the matrix cores
-(MfmaUtil) or the vector ALUs (VALUBusy) were busy, against the fraction of the
-8 TB/s the kernel's traffic past the L2s amounts to.  Compute-bound (1) when the
-compute fraction is the larger one, memory-bound (0) otherwise, unknown (-1)
-when neither reaches 5 % (a kernel that loads neither resource cannot contend
-for one).  The fractions are taken per kernel NAME, summed over all dispatches
+counter each gives: the fraction of the kernel's time the matrix cores were
+busy (MfmaUtil) against the fraction of the 8 TB/s the kernel's traffic past
+the L2s amounts to.  Compute-bound (1) when the matrix-core fraction is the
+larger one, memory-bound (0) otherwise, unknown (-1) when neither reaches 5 %
+(a kernel that loads neither resource cannot contend for one).  The vector
+ALUs' busy fraction (VALUBusy) counts address arithmetic and issue time as much
+as arithmetic -- copy, concatenation, index and pooling kernels reach 0.3-0.6 of
+it -- so it stands in for the matrix cores only for kernels whose name puts them
+in a convolution or GEMM family (MIOpen's Winograd and naive convolutions do
+their FMAs there, matrix cores idle).  The fractions are taken per kernel NAME, summed over all dispatches
 of that name in the joined iterations, weighted by duration: a 5-microsecond
 dispatch on its own says little, the family it belongs to does.  Rows whose name
 no counter run covered fall back to the name table of ``cu_need.classify`` and
@@ -132,12 +136,33 @@ def trailing_iterations(rows, n_rows, names, max_iters=5):
     return list(reversed(out))
 
 
-def classify_utilisation(memory_fraction, compute_fraction, floor=UTILISATION_FLOOR):
+def compute_family(name):
+    """True for names of convolution / GEMM / attention families: kernels whose
+    arithmetic may run on the vector ALUs with the matrix cores idle (MIOpen's
+    Winograd and naive convolutions do)."""
+    low = name.lower()
+    return any(h in low for h in cu_need.COMPUTE_HINTS)
+
+
+def classify_utilisation(memory_fraction, mfma_fraction, valu_fraction=0.0, name=None,
+                         floor=UTILISATION_FLOOR):
     """1 compute-bound, 0 memory-bound, -1 unknown: which roof the kernel is
-    closer to (see the module docstring)."""
-    if max(memory_fraction, compute_fraction) < floor:
-        return -1
-    return 1 if compute_fraction > memory_fraction else 0
+    closer to (see the module docstring).
+
+    The matrix cores are the compute roof.  Vector-ALU busy time counts address
+    arithmetic and issue time as much as arithmetic -- copy, index and pooling
+    kernels show 0.3-0.6 of it while doing next to no floating-point work (the
+    reference asks for flop/byte right of the knee, or >= 60 % utilisation:
+    roofline_analysis.py:51-66) -- so by itself it does not make a kernel
+    compute-bound.  It counts only for a kernel whose name puts it in a
+    convolution or GEMM family (``compute_family``).  Everything else is
+    memory-bound when its traffic reaches the floor, else unknown."""
+    if mfma_fraction >= floor and mfma_fraction > memory_fraction:
+        return 1
+    if (valu_fraction >= floor and valu_fraction > memory_fraction
+            and name is not None and compute_family(name)):
+        return 1
+    return 0 if memory_fraction >= floor else -1
 
 
 def merge(profile_path, rocprof_dir, out_path, use_name_hints=True, classes_out=None):
@@ -194,7 +219,7 @@ def merge(profile_path, rocprof_dir, out_path, use_name_hints=True, classes_out=
             entry["mfma_fraction"] = f["mfma_ns"] / ns
             entry["valu_fraction"] = f["valu_ns"] / ns
             entry["class"] = classify_utilisation(
-                entry["memory_fraction"], max(entry["mfma_fraction"], entry["valu_fraction"]))
+                entry["memory_fraction"], entry["mfma_fraction"], entry["valu_fraction"], name)
             entry["source"] = "counters"
         elif use_name_hints:
             entry["class"] = cu_need.classify(name)
@@ -256,7 +281,7 @@ def build_table(class_files, out_path):
     for name, a in sorted(acc.items()):
         ns = max(a["ns"], 1.0)
         mem, mfma, valu = a["memory"] / ns, a["mfma"] / ns, a["valu"] / ns
-        table[name] = {"class": classify_utilisation(mem, max(mfma, valu)),
+        table[name] = {"class": classify_utilisation(mem, mfma, valu, name),
                        "memory_fraction": round(mem, 4), "mfma_fraction": round(mfma, 4),
                        "valu_fraction": round(valu, 4), "dispatches": a["dispatches"]}
     with open(out_path, "w") as f:

@@ -66,6 +66,10 @@ def load_capture_library(path=None):
     lib.orion_client_deferred.restype = c_ulonglong
     lib.orion_client_submitted.argtypes = [c_int]
     lib.orion_client_submitted.restype = c_ulonglong
+    lib.orion_thread_time_in_calls_ns.argtypes = []
+    lib.orion_thread_time_in_calls_ns.restype = c_ulonglong
+    lib.orion_thread_calls.argtypes = []
+    lib.orion_thread_calls.restype = c_ulonglong
     lib._orion_typed = True
     return lib
 

@@ -88,20 +88,34 @@ model_names = (os.environ["FAKE_RUNNER_MODEL_NAMES"].split(",")
 assert len(model_names) == n_clients
 
 
-def write_profile(path, nk, seed):
+def write_profile(path, nk, seed, names=None):
     rng = np.random.default_rng(seed)
     with open(path, "w") as f:
         f.write("Name,Profile,Memory_footprint,SM_usage,Duration\n")
         for i in range(nk):
-            f.write(f"k{i},{int(rng.integers(-1, 2))},0,{int(rng.integers(1, 300))},"
-                    f"{int(rng.integers(5000, 60000))}\n")
+            f.write(f"{names[i] if names else f'k{i}'},{int(rng.integers(-1, 2))},0,"
+                    f"{int(rng.integers(1, 300))},{int(rng.integers(5000, 60000))}\n")
+
+
+def kernel_names(tid):
+    """FAKE_RUNNER_NAMED_PROFILE=1: profile rows carry the names of the kernels the
+    client launches (row k: saxpy for even k, sqadd for odd k).  With
+    FAKE_RUNNER_PROFILE_INSERT=r client 0's profile has one more row, named
+    fake_extra, at row r -- a profile captured with a solver the run does not use."""
+    if not os.environ.get("FAKE_RUNNER_NAMED_PROFILE"):
+        return None
+    names = ["fake_kernel_saxpy" if k % 2 == 0 else "fake_kernel_sqadd"
+             for k in range(kernels_per_iter[tid])]
+    if tid == 0 and os.environ.get("FAKE_RUNNER_PROFILE_INSERT"):
+        names.insert(int(os.environ["FAKE_RUNNER_PROFILE_INSERT"]), "fake_extra")
+    return names + ["fake_kernel_saxpy"] * 4      # spare rows: a profile may hold more
 
 
 files = []
 for c in range(n_clients):
     p = os.path.join(workdir, f"client{c}.csv")
-    write_profile(p, records_per_iter[c], c)
-    write_profile(p + ".steady", records_per_iter[c], 100 + c)   # setup_change's file
+    write_profile(p, records_per_iter[c], c, kernel_names(c))
+    write_profile(p + ".steady", records_per_iter[c], 100 + c, kernel_names(c))   # setup_change's file
     files.append(p)
 
 results = [None] * n_clients

@@ -792,7 +792,12 @@ hipError_t hipGetLastError(void) {
 }
 hipError_t hipPeekAtLastError(void) { return tl_last_error; }
 const char* hipGetErrorString(hipError_t) { return "fake hip error"; }
-const char* hipKernelNameRef(const hipFunction_t) { return "fake_kernel"; }
-const char* hipKernelNameRefByPtr(const void*, hipStream_t) { return "fake_kernel"; }
+static const char* fake_name(const void* f) {
+  if (f == (const void*)fake_kernel_saxpy) return "fake_kernel_saxpy";
+  if (f == (const void*)fake_kernel_sqadd) return "fake_kernel_sqadd";
+  return "fake_kernel";
+}
+const char* hipKernelNameRef(const hipFunction_t f) { return fake_name((const void*)f); }
+const char* hipKernelNameRefByPtr(const void* f, hipStream_t) { return fake_name(f); }
 
 }  // extern "C"

@@ -257,3 +257,39 @@ def test_more_kernels_than_the_profile_names_is_reported_at_once(tmp_path):
     assert ("client 0 submits more kernel records per iteration than the 4 its profile names"
             in proc.stderr
             or "client 0 has had a record (type" in proc.stderr), proc.stderr[-2000:]
+
+
+def test_a_count_mismatch_names_the_row_where_the_client_leaves_its_profile(tmp_path):
+    """A profile captured with one kernel more than the run launches (a different
+    convolution solver, an extra cast): the job still ends -- the count is what
+    the policy runs on -- but the report now says where the two part: the first
+    profile row whose name is not the name of the kernel launched there, and
+    both names.  (The reference spins forever, scheduler_eval.cpp:282.)"""
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), str(tmp_path),
+         "orion", "1", "20"],
+        capture_output=True, text=True, timeout=120,
+        env=dict(os.environ, FAKE_RUNNER_MISCOUNT="1", ORION_STUCK_LIMIT_S="1",
+                 FAKE_RUNNER_NAMED_PROFILE="1", FAKE_RUNNER_PROFILE_INSERT="2"))
+    assert proc.returncode != 0
+    assert "kernel count probably differs" in proc.stderr
+    assert ("client 0: first difference at profile row 2: the profile names 'fake_extra', "
+            "the client launched 'fake_kernel_saxpy'") in proc.stderr, proc.stderr[-2000:]
+
+
+def test_a_kernel_beyond_the_profile_is_named(tmp_path):
+    """The other direction: every row of the profile matches, and the client
+    launches one kernel more.  The report names that kernel."""
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "tests", "fake_runner.py"), str(tmp_path),
+         "orion", "1", "20"],
+        capture_output=True, text=True, timeout=120,
+        env=dict(os.environ, FAKE_RUNNER_MISCOUNT="-1", ORION_STUCK_LIMIT_S="2",
+                 FAKE_RUNNER_NAMED_PROFILE="1"))
+    assert proc.returncode != 0
+    if "submits more kernel records per iteration" in proc.stderr:
+        # the scheduler saw it: rows 0..3 agree, the fifth kernel (an even row: saxpy) is extra
+        assert "carry the names of profile rows 0..3" in proc.stderr, proc.stderr[-2000:]
+        assert "after the profile's last row (4 rows) it launched 'fake_kernel_saxpy'" in proc.stderr
+    else:   # the scheduler had left for the rendezvous; the waiting client reports
+        assert "client 0 has had a record (type" in proc.stderr, proc.stderr[-2000:]

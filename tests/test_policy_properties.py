@@ -23,7 +23,11 @@ bookkeeping (seen[], iteration counts, the running best-effort duration sum):
 * once the running sum of profiled durations exceeds the budget nothing
   best-effort goes out until a poll that queried events (:341-357, :363-367);
 * (this build's recorded option R1) the room of the CU budget is what the
-  high-priority op last dispatched leaves of it.
+  high-priority op last dispatched leaves of it;
+* (this build's recorded option O1) the one exception to the CU budget: a kernel
+  whose own need exceeds the device, let in as the first best-effort kernel of
+  a poll, on the smallest mask, beside an inference request whose running op
+  has the other known class, and no longer than a quarter of the budget.
 
 Profile durations are whole numbers below 2^24, so the reference's float/long
 sum is exact here.
@@ -73,11 +77,15 @@ def check_orion_invariants(obs_text, dec_text, depth):
             n, max_sms = int(p[1]), int(p[2])
             hp = n - 1
             reserve_hp = "R1" in p[4:]      # this build's option: see below
+            admit_oversized = "O1" in p[4:]
             hp_need = 0
+            hp_trains = False
         elif p[0] == "K":
             c = int(p[1])
             nk[c], max_iters[c], prof[c] = int(p[2]), int(p[3]), rows_of(p[5])
             seen[c], iters[c], event_ids[c] = 0, 0, 0
+            if c == n - 1:
+                hp_trains = bool(int(p[4]))
         elif p[0] == "X":
             c = int(p[1])
             nk[c], prof[c] = int(p[2]), rows_of(p[3])
@@ -132,7 +140,15 @@ def check_orion_invariants(obs_text, dec_text, depth):
                     throttled, running = False, 0
                 free_pass = (n == 1 or seen[hp] == 0 or cls != "k" or iters[c] <= 10
                              or hp_done)
-                if not free_pass and row is not None and hp_profile is not None:
+                if (not free_pass and row is not None and hp_profile is not None
+                        and admit_oversized and size + row[1] > max_sms):
+                    # the exception, and nothing but the exception
+                    assert size == 0 and row[1] > max_sms and not hp_trains, (line, b, size)
+                    assert row[0] != -1 and hp_profile != -1 and row[0] != hp_profile, (line, b)
+                    assert row[2] <= depth // 4, (line, b, depth)
+                    assert int(b[6]) == 0, (line, b)           # the smallest mask
+                    checked["oversized"] = checked.get("oversized", 0) + 1
+                elif not free_pass and row is not None and hp_profile is not None:
                     assert size + row[1] <= max_sms, (line, b, size)
                     if reserve_hp:      # the HP op's own CU need is taken out of the room
                         assert size + row[1] <= max(0, max_sms - hp_need), (line, b, hp_need)

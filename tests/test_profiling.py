@@ -131,15 +131,19 @@ def _counter_runs(tmp_path, kernels, iterations=2):
 
 def test_classes_from_counters_per_kernel_name(tmp_path):
     """Closed forms.  The class of a row is the class of its kernel NAME over all
-    its dispatches: traffic / time against 8000 B/ns on one side, the larger of
-    the matrix-core and vector-ALU busy fractions on the other."""
+    its dispatches: traffic / time against 8000 B/ns on one side, the matrix-core
+    busy fraction on the other; the vector-ALU busy fraction counts only for a
+    convolution or GEMM family (by name)."""
     kernels = [
         # 1 ms moving 4 GB (fetch unit 2 KiB, write unit 1 KiB): 0.5 of HBM; MFMA 10 % -> memory
         ("stream_k", 1_000_000, 1_000_000, 1_952_125, 10.0, 3.0),
         # MFMA 82 % against 0.3 of HBM -> compute
         ("gemm_k", 1_000_000, 1_000_000, 352_000, 82.0, 25.0),
-        # no matrix cores, vector ALUs 87 %, almost no traffic -> compute
+        # no matrix cores, vector ALUs 87 %, almost no traffic, and a name that says
+        # nothing: busy vector ALUs alone decide nothing -> unknown
         ("valu_k", 100_000, 10, 10, 0.0, 87.0),
+        # the same figures under a convolution's name -> compute
+        ("naive_conv_k", 100_000, 10, 10, 0.0, 87.0),
         # a tiny dispatch of stream_k with nothing measurable on its own: it takes
         # the class of its family
         ("stream_k", 2_000, 0, 0, 0.0, 0.0),
@@ -152,9 +156,9 @@ def test_classes_from_counters_per_kernel_name(tmp_path):
     rdir = _counter_runs(tmp_path, kernels)
     stats = rocprof.merge(str(prof), rdir, str(tmp_path / "out"), use_name_hints=False)
     out = [l.split(",") for l in (tmp_path / "out").read_text().splitlines()[1:]]
-    assert [int(r[1]) for r in out] == [0, 1, 1, 0, -1]
-    assert stats["from_counters"] == 5 and stats["from_names"] == 0 and stats["unknown"] == 1
-    assert abs(stats["unknown_time_fraction"] - 50_000 / 2_152_000) < 1e-9
+    assert [int(r[1]) for r in out] == [0, 1, -1, 1, 0, -1]
+    assert stats["from_counters"] == 6 and stats["from_names"] == 0 and stats["unknown"] == 2
+    assert abs(stats["unknown_time_fraction"] - 150_000 / 2_252_000) < 1e-9
     import json
     classes = json.loads((tmp_path / "out.classes.json").read_text())
     fam = classes["stream_k"]
@@ -165,7 +169,7 @@ def test_classes_from_counters_per_kernel_name(tmp_path):
     # the table built from this profile alone says the same
     table = rocprof.build_table([str(tmp_path / "out.classes.json")], str(tmp_path / "table.json"))
     assert {k: v["class"] for k, v in table.items()} == {
-        "stream_k": 0, "gemm_k": 1, "valu_k": 1, "idle_k": -1}
+        "stream_k": 0, "gemm_k": 1, "valu_k": -1, "naive_conv_k": 1, "idle_k": -1}
 
 
 def test_class_boundaries():
@@ -174,6 +178,37 @@ def test_class_boundaries():
     assert f(0.05, 0.0) == 0 and f(0.0, 0.05) == 1
     assert f(0.30, 0.30) == 0               # a tie is not "right of the knee"
     assert f(0.30, 0.31) == 1
+
+
+def test_busy_vector_alus_alone_do_not_make_a_kernel_compute_bound():
+    """VALUBusy counts address arithmetic and issue time: data movers reach
+    0.3-0.6 of it.  With the matrix cores idle it decides only for convolution
+    and GEMM families (by name); the fractions below are the ones measured on
+    the MI355X and kept in the committed table."""
+    import json
+    f = rocprof.classify_utilisation
+    table = json.load(open(cu_need.CLASS_TABLE_PATH))
+    movers = ["void at::native::CatArrayBatchedCopy", "void at::native::indexFuncLargeIndex",
+              "void at::native::max_pool_backward_nchw", "void at::native::max_pool_forward_nchw",
+              "void at::native::vectorized_layer_norm_kernel"]
+    for name in movers:
+        e = table[name]
+        assert e["valu_fraction"] > e["memory_fraction"] and e["mfma_fraction"] == 0.0, name
+        assert f(e["memory_fraction"], e["mfma_fraction"], e["valu_fraction"], name) == 0, name
+        assert e["class"] == 0, name
+    # MIOpen's Winograd and naive convolutions do their FMAs on the vector ALUs
+    for name in ("miopenSp3AsmConv_v30_3_1_gfx9_fp32_f3x2_stride2",
+                 "naive_conv_ab_nonpacked_fwd_nchw_float_double_float"):
+        e = table[name]
+        assert e["mfma_fraction"] == 0.0 and e["class"] == 1, name
+        assert f(e["memory_fraction"], e["mfma_fraction"], e["valu_fraction"], name) == 1
+    # no name, or a name outside those families: the vector ALUs do not count
+    assert f(0.28, 0.0, 0.57) == 0 and f(0.02, 0.0, 0.57, "some_copy_kernel") == -1
+    # every entry of the table carries the class its own fractions give
+    for name, e in table.items():
+        if "memory_fraction" in e:
+            assert e["class"] == f(e["memory_fraction"], e["mfma_fraction"],
+                                   e["valu_fraction"], name), name
 
 
 def test_the_flop_counter_pass_is_refused(tmp_path):
