@@ -20,12 +20,13 @@ Work done, in order (child processes first, so that this process has not touched
 the GPU when it starts them); legs after the headline are skipped, and said to
 be, when the time budget (--time-budget) would not hold them:
   1. profile both clients alone under the interception layer (gfx950 profiles);
-  2. high-priority client alone, best-effort client alone, both co-located;
+  2. best-effort client alone; then, alternating --repeats times: the
+     high-priority client alone on a plain stream with no library in the process,
+     alone behind the interception layer and the scheduler, and co-located;
   3. replay the recorded observation log through the CPU oracle and the native
      policy core: decision sequences must be identical;
   4. the same pair on plain streams with no scheduler and no interception
-     (`no_scheduler_baseline`; its isolated run is the second denominator of
-     the headline ratio);
+     (`no_scheduler_baseline`: what the scheduler is for);
   5. short legs of the other two job configurations (MobileNetV2 beside
      BERT-base training; BERT-large beside three trainers), the kernel pair
      through the scheduler, and the HIP-graph variant of the headline pair;
@@ -47,7 +48,12 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# profiles/bench_kernels_gemm8192_triad1GiB_counters.txt
+# Bytes past the L2s per launch: constants taken from the committed rocprofv3
+# FETCH_SIZE / WRITE_SIZE runs of the same kernels and shapes, not measured by
+# this program (a counter run needs the profiler around the process).
+TRAFFIC_SOURCE = ("profiles/bench_kernels_gemm8192_triad1GiB_counters.txt (rocprofv3 --pmc "
+                  "FETCH_SIZE and WRITE_SIZE runs of this kernel and shape, scaled by a copy "
+                  "kernel of known size; a constant in bench.py, not re-measured by this run)")
 GEMM_TRAFFIC_BYTES = int((786877.9 * 2.0 + 131106.5 * 1.0) * 1024)
 TRIAD_TRAFFIC_BYTES = int((1048588.2 * 2.0 + 1048576.1 * 1.0) * 1024)
 
@@ -132,7 +138,7 @@ class Legs:
         return self.deadline - time.time()
 
     def run(self, name, job, budget_ns, repeats=1, algo="orion", extra_env=None,
-            use_rocprof=False, record=False):
+            use_rocprof=False, record=False, plain_streams_too=False):
         from orion_amd import colocate
         from orion_amd.profiling import capture_profile
         if self.progress:
@@ -157,7 +163,7 @@ class Legs:
             known.append(self.be_isolated.get((capture_profile.profile_name(be), algo,
                                                tuple(sorted(env.items())))))
         res = colocate.experiment(job, algo, budget_ns, wd, env=env, repeats=repeats,
-                                  be_isolated_known=known)
+                                  be_isolated_known=known, plain_streams_too=plain_streams_too)
         for be, iso in zip(job[:-1], res["be_isolated"]):
             self.be_isolated[(capture_profile.profile_name(be), algo,
                               tuple(sorted(env.items())))] = iso
@@ -371,29 +377,40 @@ def main():
 
     if not args.kernels_only:
         t0 = time.time()
+        # every repeat: the client alone on a plain stream (no library in the
+        # process), alone behind the interception layer and the scheduler, and
+        # co-located -- so that what the path costs and what co-location costs are
+        # differences inside one alternation, not between boxes or minutes
         co = legs.run("c3", c3_job(per_run + 10), args.max_be_duration, repeats=repeats,
-                      use_rocprof=args.rocprof_profiles, record=True)
+                      use_rocprof=args.rocprof_profiles, record=True, plain_streams_too=True)
         out["value"] = co["hp_p99_ratio"]
         # one step = `per_step` requests of the co-located run
         out["ms_per_step"] = 1000.0 * per_step / co["hp_colocated"]["throughput"]
         out["hp"] = hp_summary(co)
         out["be"] = be_summary(co)[0]
         out["config"]["records_per_iteration"] = co["num_kernels"]
+        plain = co["hp_plain_isolated"]
+        out["hp"]["plain_streams_isolated_ms"] = {
+            k: plain[f"{k}_latency"] for k in ("p50", "p95", "p99")}
+        out["hp"]["requests"]["plain_streams_isolated"] = plain.get("requests")
+        out["hp"]["plain_streams_isolated_runs_p50_ms"] = [r["p50_latency"] for r in plain["runs"]] \
+            if plain.get("runs") else [plain["p50_latency"]]
+        out["hp"]["isolated_runs_p50_ms"] = [r["p50_latency"] for r in co["hp_isolated"]["runs"]] \
+            if co["hp_isolated"].get("runs") else [co["hp_isolated"]["p50_latency"]]
+        # what the path costs the client when there is nothing to schedule
+        out["hp"]["path_cost_p50_ms"] = co["hp_isolated"]["p50_latency"] - plain["p50_latency"]
+        for p in ("p50", "p99"):
+            out["hp"][f"{p}_ratio_vs_plain_streams_isolated"] = (
+                co["hp_colocated"][f"{p}_latency"] / plain[f"{p}_latency"])
         out["colocation_wall_s"] = time.time() - t0
         progress.note("replaying the recorded decisions")
         out["policy_replay"] = policy_replay(os.path.join(workdir, "c3", "colocated"))
         # The same pair with no scheduler and no interception (--algo streams):
-        # what the scheduler is for, and the second denominator of the headline
+        # what the scheduler is for
         if fits("no_scheduler_baseline", 60):
             sres = legs.run("streams", c3_job(MIN_REQUESTS + 10), args.max_be_duration,
                             algo="streams")
             out["no_scheduler_baseline"] = {**hp_summary(sres), "be": be_summary(sres)[0]}
-            plain = sres["hp_isolated"]
-            out["hp"]["plain_streams_isolated_ms"] = {
-                k: plain[f"{k}_latency"] for k in ("p50", "p95", "p99")}
-            for p in ("p50", "p99"):
-                out["hp"][f"{p}_ratio_vs_plain_streams_isolated"] = (
-                    co["hp_colocated"][f"{p}_latency"] / plain[f"{p}_latency"])
 
         short = args.short_requests
         # configs[3] and configs[4], short: a p99 over `short` requests is a few
@@ -472,13 +489,14 @@ def main():
                        "burst_achieved": gemm["burst_tflops"],
                        # bytes past the L2s per launch, from the committed rocprofv3
                        # FETCH_SIZE / WRITE_SIZE runs (scaled by a copy kernel)
-                       "traffic": GEMM_TRAFFIC_BYTES}
+                       "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE}
     tri = alone["triad"]["256"]
     out["roofline_triad"] = {"kernel": "triad_f32_kernel 3 x 1 GiB", "bound": "hbm",
                              "achieved": tri["gbs"], "peak": kp.HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": tri["gbs"] / kp.HBM_PEAK_GBS,
                              "bytes_per_launch": 12 * kp.TRIAD_ELEMS,
-                             "ms_per_launch": tri["ms"], "traffic": TRIAD_TRAFFIC_BYTES}
+                             "ms_per_launch": tri["ms"], "traffic": TRIAD_TRAFFIC_BYTES,
+                             "traffic_source": TRAFFIC_SOURCE}
     out["kernel_pair"] = {
         "workload": "configs[1]: HP bf16 GEMM 8192^3 beside BE fp32 triad over 1 GiB arrays",
         "triad_alone_gbs_by_cu_mask": {k: v["gbs"] for k, v in alone["triad"].items()},
@@ -489,6 +507,16 @@ def main():
              "triad_gbs": p["triad_gbs"],
              "triad_slowdown": p["triad_ms"] / alone["triad"][str(p["mask"])]["ms"],
              "hbm_frac_of_peak": p["triad_gbs"] / kp.HBM_PEAK_GBS} for p in pairs]}
+    if out.get("kernel_pair_scheduled"):
+        # What bounds the scheduled pair whatever the policy does: the GEMM holds
+        # the package at its power limit, so a triad confined to the smallest mask
+        # (32 of 256 CUs) already costs it this much, measured directly on two
+        # streams in this process -- beside the ratios of the scheduled legs above
+        by_mask = {str(p["mask"] or 256): p["gemm_ms"] / gemm["ms"] for p in pairs}
+        out["kernel_pair_scheduled"]["physical_bound"] = {
+            "gemm_slowdown_beside_triad_by_be_cu_mask": by_mask,
+            "note": "closed-loop GEMM requests beside the triad cannot do better than the "
+                    "32-CU figure: compare it with closed_loop.hp_p99_ratio"}
     if args.kernels_only:
         out["value"] = gemm["tflops"]
         out["metric"] = "kernel pair only (profiler run)"

@@ -106,6 +106,7 @@ def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
                 loss.backward()
                 optimizer.step()
                 state["loss"] = loss
+                cc.keep_loss(state, batch_idx, loss)
             else:
                 with torch.no_grad():
                     out = model(input_ids=ids, token_type_ids=seg, attention_mask=mask)
@@ -119,6 +120,7 @@ def bert_loop(batchsize, train, num_iters, rps, uniform, dummy_data, local_rank,
                            os.path.join(save_dir, f"client_{tid}_output.pt"))
             if "loss" in state:
                 res["final_loss"] = float(state["loss"].detach().float().cpu())
+            res.update(cc.loss_checkpoint_report(state))
             return res
 
         with cc.uncaptured(backend):

@@ -72,6 +72,31 @@ def latency_summary(timings, batch_idx, total_time, train, drop=WARMUP_ITERS):
     return {"throughput": throughput}
 
 
+def loss_checkpoints():
+    """ORION_LOSS_AT_ITERATION=N[,M...]: a training client keeps the loss tensors
+    of these scheduled iterations (no copy, no wait: the tensors are simply not
+    let go) and reports their values after the run.  The loss of iteration N
+    depends on every parameter update before it, so two runs of the same client
+    -- alone, and beside other clients -- can be compared at fixed points although
+    they run for different numbers of iterations.  Empty: off."""
+    text = os.environ.get("ORION_LOSS_AT_ITERATION", "")
+    return {int(t) for t in text.split(",") if t.strip()}
+
+
+def keep_loss(state, batch_idx, loss):
+    if batch_idx in loss_checkpoints():
+        state.setdefault("loss_at", {})[batch_idx] = loss     # read back after the run
+
+
+def loss_checkpoint_report(state):
+    """``loss_at_iteration``: iteration -> [value, bit pattern of the fp32 value]."""
+    out = {}
+    for it, loss in sorted(state.get("loss_at", {}).items()):
+        value = loss.detach().float().cpu()
+        out[str(it)] = [float(value), int(value.view(torch.int32))]
+    return {"loss_at_iteration": out} if out else {}
+
+
 def brief(data):
     """A result without its per-request list, for the one-line report."""
     return {k: v for k, v in data.items() if k != "latencies_ms"}

@@ -5,7 +5,7 @@ Counterpart of the reference's ``imagenet_loop``
 (benchmarking/benchmark_suite/train_imagenet.py:71-241): same keyword
 arguments, same loop and barrier protocol, same ``client_{tid}.json``.  Extra,
 optional keys of a job's ``args``: ``dtype`` ("fp32" | "bf16"), ``momentum``,
-``seed``, ``deterministic``.  Synthetic data follows the job description: images N(0,1), labels
+``lr`` (0.1, the reference's, :116), ``seed``, ``deterministic``, ``hip_graph``.  Synthetic data follows the job description: images N(0,1), labels
 uniform over the classes (the reference uses U(0,1) images and all-ones labels,
 :36-37).
 """
@@ -40,7 +40,7 @@ class DummyDataLoader:
 def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                   dummy_data, local_rank, barriers, client_barrier, tid,
                   input_file="", dtype="fp32", momentum=0.9, seed=42,
-                  deterministic=False, hip_graph=False):
+                  deterministic=False, hip_graph=False, lr=0.1):
     cc.seed_everything(seed)
     if deterministic:
         # keep MIOpen off solvers that accumulate with atomics (split-K), whose
@@ -72,7 +72,7 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
             model = model.to(device)
             if train:
                 model.train()
-                optimizer = torch.optim.SGD(model.parameters(), lr=0.1, momentum=momentum)
+                optimizer = torch.optim.SGD(model.parameters(), lr=lr, momentum=momentum)
                 criterion = torch.nn.CrossEntropyLoss().to(device)
             else:
                 model.eval()
@@ -92,6 +92,7 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                 loss.backward()
                 optimizer.step()
                 state["loss"] = loss
+                cc.keep_loss(state, batch_idx, loss)
             elif "graph" in state:
                 # one copy record and one graph record per request
                 state["graph_in"].copy_(data, non_blocking=True)
@@ -110,6 +111,7 @@ def imagenet_loop(model_name, batchsize, train, num_iters, rps, uniform,
                            os.path.join(save_dir, f"client_{tid}_output.pt"))
             if "loss" in state:
                 out["final_loss"] = float(state["loss"].detach().float().cpu())
+            out.update(cc.loss_checkpoint_report(state))
             return out
 
         with cc.uncaptured(backend):

@@ -88,7 +88,7 @@ def pooled(runs):
 
 def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
                be_isolated_iters=60, env=None, skip_isolated=False, repeats=1,
-               be_isolated_known=None):
+               be_isolated_known=None, plain_streams_too=False):
     """Runs the high-priority client alone, every best-effort client alone, and
     the whole job; reports the high-priority client's latency ratios and what
     each best-effort client keeps of its own throughput.
@@ -100,7 +100,12 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
 
     ``be_isolated_known``: one entry per best-effort client, a result of an
     earlier isolated run of the same client under the same settings, or None to
-    measure it here."""
+    measure it here.
+
+    ``plain_streams_too``: every repeat also runs the high-priority client alone
+    on a plain stream, with no scheduler and no interception library in the
+    process (``hp_plain_isolated`` in the result): what the path itself costs
+    the client, measured in the same alternation as everything else."""
     workdir = workdir or tempfile.mkdtemp(prefix="orion_colocate_")
     hp = job[-1]
     result = {"algo": algo, "max_be_duration_ns": max_be_duration, "workdir": workdir}
@@ -117,9 +122,14 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
             result["be_isolated"].append(
                 run_job([entry], algo, os.path.join(workdir, f"iso_be{k}"),
                         max_be_duration, env=env)[0])
-    iso_runs, co_runs = [], []
+    iso_runs, co_runs, plain_runs = [], [], []
     for rep in range(repeats):
         tag = f"_{rep}" if repeats > 1 else ""
+        if plain_streams_too:
+            plain = copy.deepcopy(hp)
+            plain["kernel_file"], plain["num_kernels"] = "", 0
+            plain_runs.append(run_job([plain], "streams", os.path.join(workdir, "plain_hp" + tag),
+                                      max_be_duration)[0])
         if not skip_isolated:
             iso_runs.append(run_job([copy.deepcopy(hp)], algo,
                                     os.path.join(workdir, "iso_hp" + tag),
@@ -131,6 +141,8 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
             co_runs.append(run_job(copy.deepcopy(job), algo,
                                    os.path.join(workdir, "colocated" + tag),
                                    max_be_duration, env=co_env))
+    if plain_runs:
+        result["hp_plain_isolated"] = pooled(plain_runs)
     if iso_runs:
         result["hp_isolated"] = pooled(iso_runs)
     if co_runs:
