@@ -133,6 +133,37 @@ void pin_caller(int slot, pid_t tid) {
   if (sched_setaffinity(0, sizeof one, &one) == 0) g_pin.tid[slot] = tid;
 }
 
+// Threads that are no client's own but issue work on a client's behalf (calls
+// routed by the stream they name: a framework's autograd worker) are put on that
+// client's CPU the first time they do, once per job (reference: the lazily
+// registered backward threads of utils_interc.cpp:28-49 share their client's
+// CPU); the client waits while such a thread works for it.
+struct HelperPin {
+  pid_t tid;
+  int cpu;
+  cpu_set_t before;
+};
+std::mutex g_helper_lock;
+std::vector<HelperPin> g_helpers;
+thread_local uint32_t tl_helper_epoch = 0;
+
+void pin_helper(int client) {
+  if (!g_pin.on || !g_pin.clients) return;
+  const uint32_t e = g_state.epoch.load(std::memory_order_acquire);
+  if (tl_helper_epoch == e) return;      // placed (or tried) once per job
+  tl_helper_epoch = e;
+  HelperPin h;
+  h.tid = (pid_t)syscall(SYS_gettid);
+  h.cpu = g_pin.cpus[client + 1];
+  if (sched_getaffinity(0, sizeof(cpu_set_t), &h.before) != 0) return;
+  cpu_set_t one;
+  CPU_ZERO(&one);
+  CPU_SET(h.cpu, &one);
+  if (sched_setaffinity(0, sizeof one, &one) != 0) return;
+  std::lock_guard<std::mutex> hold(g_helper_lock);
+  g_helpers.push_back(h);
+}
+
 void pinning_undo() {
   for (int s = 0; s <= kMaxClients; ++s) {
     if (g_pin.tid[s] == 0) continue;
@@ -140,6 +171,10 @@ void pinning_undo() {
     (void)sched_setaffinity(g_pin.tid[s], sizeof(cpu_set_t), &g_pin.before[s]);
     g_pin.tid[s] = 0;
   }
+  std::lock_guard<std::mutex> hold(g_helper_lock);
+  for (const HelperPin& h : g_helpers)
+    (void)sched_setaffinity(h.tid, sizeof(cpu_set_t), &h.before);
+  g_helpers.clear();
 }
 
 int lookup_thread() {
@@ -167,7 +202,10 @@ inline int client_for_call(hipStream_t stream) {
   if ((pid_t)syscall(SYS_gettid) == g_state.scheduler_tid) return kNotClient;
   for (int i = 0; i < g_state.num_clients; ++i)
     for (auto& s : g_state.channels[i].own_streams)
-      if (s.load(std::memory_order_relaxed) == stream) return i;
+      if (s.load(std::memory_order_relaxed) == stream) {
+        pin_helper(i);
+        return i;
+      }
   return kNotClient;
 }
 
@@ -401,6 +439,9 @@ int orion_pinned_cpu(void) {
   const pid_t tid = (pid_t)syscall(SYS_gettid);
   for (int s = 0; s <= kMaxClients; ++s)
     if (g_pin.tid[s] == tid) return g_pin.cpus[s + 1];
+  std::lock_guard<std::mutex> hold(g_helper_lock);
+  for (const HelperPin& h : g_helpers)
+    if (h.tid == tid) return h.cpu;
   return -1;
 }
 

@@ -251,7 +251,10 @@ class LiveHost : public PolicyHost {
     }
     client_stream_[(size_t)d.client] = stream;
     cur_cu_slot_[(size_t)d.client] = slot;
-    ch.last_stream.store(stream, std::memory_order_release);
+    // written only when it changes: the line also holds what the client reads on
+    // every call (direct_stream), and a store here would take it away each time
+    if (ch.last_stream.load(std::memory_order_relaxed) != stream)
+      ch.last_stream.store(stream, std::memory_order_release);
 
     // The outcome goes to the waiting caller's own storage (Record::cell), and
     // must be there before head moves: from then on the slot is the client's

@@ -24,6 +24,7 @@ CHILD = textwrap.dedent("""
         tids[i] = threading.get_native_id()
         go.wait(); armed.wait()
         seen[("idx", i)] = cap.orion_client_index()
+        seen[("cpu", i)] = cap.orion_pinned_cpu()
         cap.orion_register_stream(STREAM_OF[i])
         cap.orion_thread_passthrough(1)
         seen[("bypass", i)] = cap.orion_client_index()
@@ -45,6 +46,9 @@ CHILD = textwrap.dedent("""
         seen["stranger"] = [cap.orion_client_index(), cap.orion_client_of_stream(None),
                             cap.orion_client_of_stream(0x9999)] + [
                             cap.orion_client_of_stream(s) for s in STREAM_OF.values()]
+        # the first client it worked for (client 0) decides where it runs
+        import os
+        seen["stranger_cpu"] = [cap.orion_pinned_cpu(), sorted(os.sched_getaffinity(0))]
         cap.orion_register_thread(1)          # an adopted helper thread
         seen["adopted"] = [cap.orion_client_index(), cap.orion_client_of_stream(0x1000)]
         done.wait()
@@ -82,6 +86,14 @@ def test_thread_and_stream_identity():
     assert seen["stranger"][3:] == [0, 1, 2]
     # an adopted thread is its client whatever stream it names
     assert seen["adopted"] == [1, 1]
+    # a thread that works for a client by naming its stream runs on that client's
+    # CPU from then on (reference: utils_interc.cpp:28-49), when threads are pinned
+    cpu0 = seen[str(("cpu", 0))]
+    if cpu0 >= 0:
+        assert seen["stranger_cpu"] == [cpu0, [cpu0]]
+        assert len({seen[str(("cpu", i))] for i in range(3)}) == 3
+    else:
+        assert seen["stranger_cpu"][0] < 0
 
 
 def test_rearming_remaps_cached_threads():
