@@ -15,13 +15,15 @@ Both logs are line-based text, shared with the native core
 (orion_amd/csrc/policy/obslog.h):
 
 observation log
-    ``J <n> <max_sms> <place_masks comma list> [L1] [R1] [O1]``  job header (L1: long
+    ``J <n> <max_sms> <place_masks comma list> [L1] [R1] [O1] [T1]``  job header (L1: long
                                                     best-effort kernels confined; R1:
                                                     the high-priority op's CU need
                                                     is reserved; O1: short kernels of
                                                     the other class whose CU need
                                                     exceeds the device go in alone,
-                                                    on the smallest mask)
+                                                    on the smallest mask; T1: the
+                                                    duration throttle lets go at its
+                                                    half-way mark)
     ``K <client> <num_kernels> <num_iters> <train 0|1> <profile path>``
     ``X <client> <num_kernels> <profile path>``      setup_change
     ``S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>``
@@ -105,11 +107,12 @@ class RecordingEnv(po.Env):
 
     # structure markers -------------------------------------------------
     def header(self, max_sms, clients, confine_long=False, reserve_hp=False,
-               admit_oversized=False):
+               admit_oversized=False, sliding_throttle=False):
         self.confine_long = bool(confine_long)
         self.obs.append(f"J {self.n} {max_sms} " + ",".join(map(str, self.masks))
                         + (" L1" if confine_long else "") + (" R1" if reserve_hp else "")
-                        + (" O1" if admit_oversized else ""))
+                        + (" O1" if admit_oversized else "")
+                        + (" T1" if sliding_throttle else ""))
         for i, (nk, ni, train, path) in enumerate(clients):
             self.obs.append(f"K {i} {nk} {ni} {int(bool(train))} {path}")
 
@@ -182,6 +185,10 @@ class RecordingEnv(po.Env):
         self._dec.append(f"D {client} {owner} {cls} {op_index} {event_slot} "
                          f"{cu_slot}")
         self.inner.dispatch(client, owner, cls, op_index, event_slot)
+
+    def mark(self, owner, index):
+        if hasattr(self.inner, "mark"):
+            self.inner.mark(owner, index)
 
     def iteration_done(self, client, iteration):
         self._dec.append(f"F {client} {iteration}")
@@ -259,7 +266,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
     oracle = None
     rec = None
     n = max_sms = masks = None
-    confine_long = reserve_hp = admit_oversized = False
+    confine_long = reserve_hp = admit_oversized = sliding_throttle = False
     clients = {}
     lines = obs_text.splitlines()
     i = 0
@@ -269,10 +276,11 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
         if tag == "J":
             n, max_sms = int(parts[1]), int(parts[2])
             masks = [int(x) for x in parts[3].split(",")]
-            _ensure(set(parts[4:]) <= {"L1", "R1", "O1"} and len(parts) <= 7,
-                    "J: 3 fields and optional L1 / R1 / O1")
+            _ensure(set(parts[4:]) <= {"L1", "R1", "O1", "T1"} and len(parts) <= 8,
+                    "J: 3 fields and optional L1 / R1 / O1 / T1")
             confine_long, reserve_hp = "L1" in parts[4:], "R1" in parts[4:]
             admit_oversized = "O1" in parts[4:]
+            sliding_throttle = "T1" in parts[4:]
         elif tag == "K":
             clients[int(parts[1])] = (int(parts[2]), int(parts[3]),
                                       bool(int(parts[4])), " ".join(parts[5:]))
@@ -289,7 +297,7 @@ def replay(obs_text, load_profile=po.parse_profile, sequential_fix=True, mark_po
                     [load_profile(c[3]) for c in order], [c[0] for c in order],
                     [c[1] for c in order], [c[2] for c in order], max_sms,
                     sequential_fix=sequential_fix, reserve_hp=reserve_hp,
-                    admit_oversized=admit_oversized)
+                    admit_oversized=admit_oversized, sliding_throttle=sliding_throttle)
             polls = []
             i += 1
             while lines[i] != "E":

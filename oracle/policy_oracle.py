@@ -150,6 +150,9 @@ class Env:
     def set_stop(self, client):            # client_stop[k] = true
         raise NotImplementedError
 
+    def mark(self, owner, index):          # sliding_throttle only: a later
+        pass                               # event_done(owner, index) will come
+
 
 class PolicyOracle:
     """State that the reference keeps in file-scope globals
@@ -157,7 +160,15 @@ class PolicyOracle:
     ``schedule`` calls: seen, event_ids, cur_iters, penalty, profiles."""
 
     def __init__(self, profiles, num_kernels, num_iters, is_train, max_sms=80,
-                 sequential_fix=False, reserve_hp=False, admit_oversized=False):
+                 sequential_fix=False, reserve_hp=False, admit_oversized=False,
+                 sliding_throttle=False):
+        # sliding_throttle (not in the reference, whose throttle :342-359 lets
+        # go only when every best-effort stream has drained): when the duration
+        # sum first passes depth // 2 the latest kernel of every best-effort
+        # client is remembered (a mark) together with the sum; while throttled
+        # the marks are asked about too, and once all have completed that part
+        # of the sum is taken off and admission goes on.
+        self.sliding_throttle = bool(sliding_throttle)
         # admit_oversized (not in the reference, whose CU clause :339-340 can
         # never admit a kernel whose un-clipped need exceeds max_sms while a
         # high-priority inference request is in flight): such a kernel goes in
@@ -312,6 +323,9 @@ class PolicyOracle:
             update_start = INT_MAX
         polls = 0
         hp_need = 0
+        mark_index = [-1] * n        # sliding_throttle: see __init__
+        mark_valid = False
+        mark_sum = 0
 
         while True:                                          # :277
             env.begin_poll()
@@ -379,6 +393,21 @@ class PolicyOracle:
                             large_found = False
                             total = 0
                             self._changed = True
+                            mark_valid = False
+                        elif self.sliding_throttle and mark_valid:
+                            half = True
+                            for k in range(n - 1):
+                                if mark_index[k] >= 0:
+                                    if not env.event_done(k, mark_index[k]):
+                                        half = False
+                                        break
+                            if half:
+                                total = max(0, total - mark_sum)
+                                mark_valid = False
+                                large_found = False
+                                self._changed = True
+                            else:
+                                go = False
                         else:
                             go = False
                     if go:                                   # :360-375
@@ -392,6 +421,14 @@ class PolicyOracle:
                             large_found = True               # :366-368
                         self._dispatch(env, j, j, cls, oversized)
                         start = j                            # :374
+                        if (self.sliding_throttle and not mem_op and not mark_valid
+                                and total > depth // 2):
+                            for k in range(n - 1):
+                                mark_index[k] = self.event_ids[k] - 1
+                                if mark_index[k] >= 0:
+                                    env.mark(k, mark_index[k])
+                            mark_sum = total
+                            mark_valid = True
 
             finished = 0                                     # :380
             for i in range(n):
@@ -410,6 +447,7 @@ class PolicyOracle:
                         if seq:
                             self.event_ids[0] = 0
                         self.event_ids[i] = 0
+                        mark_index[i] = -1       # nothing of it is outstanding
                         env.iteration_done(i, self.cur_iters[i])
                         self.cur_iters[i] += 1
                         self._changed = True

@@ -21,13 +21,14 @@ void appendf(std::string* s, const char* fmt, ...) {
 }  // namespace
 
 void Recorder::header(int max_sms, const std::vector<int>& masks, bool confine_long,
-                      bool reserve_hp, bool admit_oversized) {
+                      bool reserve_hp, bool admit_oversized, bool sliding_throttle) {
   appendf(&obs_, "J %d %d ", n_, max_sms);
   for (size_t i = 0; i < masks.size(); ++i)
     appendf(&obs_, i ? ",%d" : "%d", masks[i]);
   if (confine_long) obs_ += " L1";  // long best-effort kernels are confined
   if (reserve_hp) obs_ += " R1";    // the high-priority op's CU need is reserved
   if (admit_oversized) obs_ += " O1";  // oversized short kernels of the other class go in alone
+  if (sliding_throttle) obs_ += " T1"; // the throttle lets go at its half-way mark
   obs_ += '\n';
 }
 
@@ -235,6 +236,7 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
 
   int n = 0, max_sms = 0;
   bool confine_long = false, reserve_hp = false, admit_oversized = false;
+  bool sliding_throttle = false;
   std::vector<int> masks;
   std::vector<ClientDesc> clients;
   Policy* policy = nullptr;
@@ -248,16 +250,17 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
     if (l.empty()) continue;
     const char tag = l[0];
     if (tag == 'J') {
-      auto p = split(l, ' ', 7);
-      bool options_ok = p.size() >= 4 && p.size() <= 7;
+      auto p = split(l, ' ', 9);
+      bool options_ok = p.size() >= 4 && p.size() <= 8;
       for (size_t k = 4; options_ok && k < p.size(); ++k) {
         if (p[k] == "L1") confine_long = true;
         else if (p[k] == "R1") reserve_hp = true;
         else if (p[k] == "O1") admit_oversized = true;
+        else if (p[k] == "T1") sliding_throttle = true;
         else options_ok = false;
       }
       if (!options_ok) {
-        ok = bad(i, "J needs 3 fields and optional L1 / R1 / O1");
+        ok = bad(i, "J needs 3 fields and optional L1 / R1 / O1 / T1");
         break;
       }
       n = atoi(p[1].c_str());
@@ -307,7 +310,8 @@ bool replay_observations(const std::string& obs, bool sequential_fix,
         }
         if (!ok) break;
         policy = new Policy(std::move(profs), nk, ni, tr, max_sms, masks,
-                            sequential_fix, confine_long, reserve_hp, admit_oversized);
+                            sequential_fix, confine_long, reserve_hp, admit_oversized,
+                            sliding_throttle);
       }
       ScheduleArgs a;
       a.warmup = atoi(p[1].c_str()) != 0;

@@ -9,11 +9,13 @@
 //
 // Line formats (text, one record per line):
 //   observation log
-//     J <n> <max_sms> <cu mask sizes, comma separated> [L1] [R1] [O1]
+//     J <n> <max_sms> <cu mask sizes, comma separated> [L1] [R1] [O1] [T1]
 //       (L1: long best-effort kernels are confined to a partial mask;
 //        R1: the high-priority op's own CU need is reserved;
 //        O1: short best-effort kernels of the opposite class whose CU need
-//            exceeds the device are admitted alone on the smallest mask)
+//            exceeds the device are admitted alone on the smallest mask;
+//        T1: the duration throttle lets go when the work outstanding at its
+//            half-way mark has completed, not only when every stream is empty)
 //     K <client> <num_kernels> <num_iters> <train 0|1> <profile path>
 //     X <client> <num_kernels> <profile path>               setup_change
 //     S <warmup 0|1> <warmup_iters> <algo> <depth> <hp_limit> <update_start>
@@ -43,7 +45,8 @@ class Recorder : public PolicyHost {
   void set_mark_polls(bool on) { mark_polls_ = on; }
 
   void header(int max_sms, const std::vector<int>& masks, bool confine_long = false,
-              bool reserve_hp = false, bool admit_oversized = false);
+              bool reserve_hp = false, bool admit_oversized = false,
+              bool sliding_throttle = false);
   void client(int idx, int num_kernels, int num_iters, bool train,
               const std::string& profile_path);
   void setup_change(int client, int num_kernels, const std::string& path);
@@ -52,6 +55,7 @@ class Recorder : public PolicyHost {
 
   void begin_poll() override;
   void end_poll(bool effective) override;
+  void mark(int owner, int index) override { inner_->mark(owner, index); }
   bool stop_ack(int client) override;
   int peek(int client) override;
   bool event_done(int owner, int index) override;

@@ -135,7 +135,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
                std::vector<int> num_kernels, std::vector<int> num_iters,
                std::vector<bool> is_train, int max_sms,
                std::vector<int> cu_masks, bool sequential_fix, bool confine_long,
-               bool reserve_hp, bool admit_oversized)
+               bool reserve_hp, bool admit_oversized, bool sliding_throttle)
     : n_((int)profiles.size()),
       ops_(std::move(profiles)),
       num_kernels_(std::move(num_kernels)),
@@ -147,6 +147,7 @@ Policy::Policy(std::vector<std::vector<OpInfo>> profiles,
       confine_long_(confine_long),
       reserve_hp_(reserve_hp),
       admit_oversized_(admit_oversized),
+      sliding_throttle_(sliding_throttle),
       seen_(n_, 0),
       event_ids_(n_, 0),
       cur_iters_(n_, 0),
@@ -305,6 +306,11 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
   std::vector<int> heads(n);
   int64_t polls = 0;
   int hp_need = 0;  // CU need of the high-priority op last dispatched (reserve_hp_)
+  // sliding_throttle_: per best-effort client the kernel that was its latest when
+  // the sum passed half the budget (-1: none), and the sum at that moment
+  std::vector<int> mark_index(n, -1);
+  bool mark_valid = false;
+  long mark_sum = 0;
 
   for (;;) {
     host.begin_poll();
@@ -374,6 +380,26 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
             large_found = false;
             sum = 0;
             changed_ = true;
+            mark_valid = false;
+          } else if (sliding_throttle_ && mark_valid) {
+            bool half = true;
+            for (int k = 0; k < n - 1; ++k) {
+              if (mark_index[k] >= 0 && !host.event_done(k, mark_index[k])) {
+                half = false;
+                break;
+              }
+            }
+            if (half) {
+              // everything dispatched up to the marks has completed
+              sum -= mark_sum;
+              if (sum < 0) sum = 0;
+              mark_valid = false;
+              large_found = false;
+              changed_ = true;
+            } else {
+              go = false;
+              outcome = ADM_THROTTLED;
+            }
           } else {
             go = false;
             outcome = ADM_THROTTLED;
@@ -387,6 +413,14 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
             large_found = true;
           dispatch(host, j, j, cls, oversized);
           start = j;
+          if (sliding_throttle_ && !mem_op && !mark_valid && sum > args.depth / 2) {
+            for (int k = 0; k < n - 1; ++k) {
+              mark_index[k] = event_ids_[k] - 1;
+              if (mark_index[k] >= 0) host.mark(k, mark_index[k]);
+            }
+            mark_sum = sum;
+            mark_valid = true;
+          }
         }
       }
     }
@@ -407,6 +441,7 @@ int64_t Policy::schedule(PolicyHost& host, const ScheduleArgs& args) {
           seen_[i] = 0;
           if (is_seq) event_ids_[0] = 0;
           event_ids_[i] = 0;
+          mark_index[i] = -1;  // a completed iteration has nothing outstanding
           host.iteration_done(i, cur_iters_[i]);
           cur_iters_[i] += 1;
           changed_ = true;

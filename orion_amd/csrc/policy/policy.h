@@ -88,6 +88,10 @@ class PolicyHost {
   virtual void dispatch(const Dispatch& d) = 0;
   virtual void iteration_done(int client, int iteration) = 0;
   virtual void set_stop(int client) = 0;
+  // Option sliding_throttle only: the policy will ask event_done(owner, index)
+  // about this kernel later although newer ones will have been dispatched by
+  // then; index is the owner's latest kernel at the time of the call.
+  virtual void mark(int /*owner*/, int /*index*/) {}
 };
 
 // Per best-effort client, counted once per poll in which the client had a record
@@ -124,7 +128,7 @@ class Policy {
          std::vector<bool> is_train, int max_sms,
          std::vector<int> cu_masks, bool sequential_fix,
          bool confine_long = false, bool reserve_hp = false,
-         bool admit_oversized = false);
+         bool admit_oversized = false, bool sliding_throttle = false);
 
   void setup_change(int client, std::vector<OpInfo> ops, int num_kernels);
 
@@ -182,6 +186,18 @@ class Policy {
   // duration is at most a quarter of the duration budget; it goes to the
   // smallest mask.  Everything else is the reference's rule.
   bool admit_oversized_;
+  // Throttle option (not in the reference).  The reference stops admitting
+  // best-effort kernels once the sum of their profiled durations exceeds the
+  // budget and starts again only when EVERY best-effort stream has drained
+  // (scheduler_eval.cpp:342-359, :366-368): the GPU's best-effort queue runs
+  // empty every `budget` nanoseconds of work, and refills at the client's own
+  // pace.  With the option the policy also remembers, when the sum first passes
+  // half the budget, the latest kernel of every best-effort client (a mark) and
+  // the sum at that point; while throttled it asks about the marks as well, and
+  // once they have all completed it takes that part of the sum off and goes on
+  // -- the outstanding work stays bounded by the budget, as in the reference,
+  // but no longer has to fall to zero.
+  bool sliding_throttle_;
   // survive between schedule() calls, like the reference's globals
   std::vector<int> seen_;
   std::vector<int> event_ids_;

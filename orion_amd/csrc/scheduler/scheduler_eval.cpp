@@ -92,6 +92,8 @@ class LiveHost : public PolicyHost {
     streams_.resize((size_t)n);
     last_event_.assign((size_t)n, nullptr);
     chain_event_.assign((size_t)n, nullptr);
+    mark_event_.assign((size_t)n, nullptr);
+    mark_slot_.assign((size_t)n, -1);
     last_recorded_.assign((size_t)n, true);
     last_slot_.assign((size_t)n, -1);
     last_kernel_stream_.assign((size_t)n, nullptr);
@@ -113,6 +115,7 @@ class LiveHost : public PolicyHost {
         if (s) (void)hip_->hipStreamDestroy(s);
     for (hipEvent_t e : last_event_) if (e) (void)hip_->hipEventDestroy(e);
     for (hipEvent_t e : chain_event_) if (e) (void)hip_->hipEventDestroy(e);
+    for (hipEvent_t e : mark_event_) if (e) (void)hip_->hipEventDestroy(e);
     if (update_event_) (void)hip_->hipEventDestroy(update_event_);
   }
 
@@ -193,6 +196,8 @@ class LiveHost : public PolicyHost {
     }
     if (owner == update_owner_ && index == update_slot_ && update_valid_)
       return hip_->hipEventQuery(update_event_) == hipSuccess;
+    if (index == mark_slot_[(size_t)owner])
+      return hip_->hipEventQuery(mark_event_[(size_t)owner]) == hipSuccess;
     // An index the policy can only reach after the op completed long ago.
     return true;
   }
@@ -322,6 +327,7 @@ class LiveHost : public PolicyHost {
     if (hipStream_t direct = ch.direct_stream.load(std::memory_order_relaxed))
       (void)hip_->hipStreamSynchronize(direct);
     ch.released_iters.store((int64_t)iteration + 1, std::memory_order_release);
+    mark_slot_[(size_t)client] = -1;
     const float ms = (float)iteration_us(client) / 1000.0f;
     durations_ms_[(size_t)client].push_back(ms);
     start_pending_[(size_t)client] = true;
@@ -392,6 +398,18 @@ class LiveHost : public PolicyHost {
     cap_->channels[client].stop.store(1, std::memory_order_release);
   }
 
+  // The policy will ask about this kernel after newer ones have gone out: an
+  // event of its own, recorded now, behind the owner's latest kernel.
+  void mark(int owner, int index) override {
+    mark_slot_[(size_t)owner] = -1;
+    if (index < 0 || index != last_slot_[(size_t)owner] ||
+        last_kernel_stream_[(size_t)owner] == nullptr)
+      return;   // nothing of the owner's is in flight under that index: "done"
+    check(hip_->hipEventRecord(mark_event_[(size_t)owner], last_kernel_stream_[(size_t)owner]),
+          "hipEventRecord(mark)");
+    mark_slot_[(size_t)owner] = index;
+  }
+
  private:
   // The reference spins forever when a client's kernel count disagrees with its
   // profile, or when a client dies mid-iteration (scheduler_eval.cpp:282, :389).
@@ -436,6 +454,8 @@ class LiveHost : public PolicyHost {
             "hipEventCreateWithFlags");
       check(hip_->hipEventCreateWithFlags(&chain_event_[(size_t)c], hipEventDisableTiming),
             "hipEventCreateWithFlags");
+      check(hip_->hipEventCreateWithFlags(&mark_event_[(size_t)c], hipEventDisableTiming),
+            "hipEventCreateWithFlags");
       if (is_hp) {
         hipStream_t s = nullptr;
         check(hip_->hipStreamCreateWithFlags(&s, hipStreamNonBlocking),
@@ -474,7 +494,8 @@ class LiveHost : public PolicyHost {
   const HipApi* hip_;
   CaptureState* cap_;
   std::vector<std::vector<hipStream_t>> streams_;   // [client][cu slot]
-  std::vector<hipEvent_t> last_event_, chain_event_;
+  std::vector<hipEvent_t> last_event_, chain_event_, mark_event_;
+  std::vector<int> mark_slot_;   // event index each mark event stands for, -1 = none
   std::vector<char> last_recorded_;
   std::vector<int> last_slot_;
   std::vector<hipStream_t> last_kernel_stream_, client_stream_;
@@ -627,8 +648,13 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** models,
   // CU need exceeds the device in alone, on the smallest mask (see policy.h).
   const bool admit_oversized = getenv("ORION_ADMIT_OVERSIZED") &&
                                atoi(getenv("ORION_ADMIT_OVERSIZED")) != 0;
+  // Throttle option: let go at the half-way mark instead of waiting for every
+  // best-effort stream to run empty (see policy.h).
+  const bool sliding_throttle = getenv("ORION_SLIDING_THROTTLE") &&
+                                atoi(getenv("ORION_SLIDING_THROTTLE")) != 0;
   g.policy.reset(new Policy(std::move(profiles), nk, ni, g.is_train, max_sms, g.masks,
-                            !as_written, confine_long, reserve_hp, admit_oversized));
+                            !as_written, confine_long, reserve_hp, admit_oversized,
+                            sliding_throttle));
   g.host.reset(new LiveHost(num_clients, cus, g.masks));
   g.host->set_policy(g.policy.get());
   g.recorder.reset();
@@ -637,7 +663,8 @@ void setup(void* /*scheduler*/, int num_clients, int* tids, char** models,
     if (*dir) {
       g.record_dir = dir;
       g.recorder.reset(new Recorder(g.host.get(), num_clients));
-      g.recorder->header(max_sms, g.masks, confine_long, reserve_hp, admit_oversized);
+      g.recorder->header(max_sms, g.masks, confine_long, reserve_hp, admit_oversized,
+                         sliding_throttle);
       for (int i = 0; i < num_clients; ++i)
         g.recorder->client(i, nk[(size_t)i], ni[(size_t)i], g.is_train[(size_t)i], files[i]);
       // start both logs afresh

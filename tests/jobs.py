@@ -94,6 +94,7 @@ def make_job(tmp_path, seed, n_clients=2, algo=po.ALGO_ORION, hp_train=False,
     job.confine_long = rng.random() < 0.5
     job.reserve_hp = rng.random() < 0.4
     job.admit_oversized = rng.random() < 0.4
+    job.sliding_throttle = rng.random() < 0.4
     return job
 
 
@@ -103,7 +104,8 @@ def run_oracle(job, max_polls=3_000_000):
                              max_sms=job.max_sms,
                              sequential_fix=job.sequential_fix,
                              reserve_hp=getattr(job, "reserve_hp", False),
-                             admit_oversized=getattr(job, "admit_oversized", False))
+                             admit_oversized=getattr(job, "admit_oversized", False),
+                             sliding_throttle=getattr(job, "sliding_throttle", False))
     clients = []
     for c in range(job.n):
         first, main = job.traces[c]
@@ -123,7 +125,8 @@ def run_oracle(job, max_polls=3_000_000):
                               job.paths[c]) for c in range(job.n)],
                confine_long=getattr(job, "confine_long", False),
                reserve_hp=getattr(job, "reserve_hp", False),
-               admit_oversized=getattr(job, "admit_oversized", False))
+               admit_oversized=getattr(job, "admit_oversized", False),
+               sliding_throttle=getattr(job, "sliding_throttle", False))
     changes = {1: [(c, po.parse_profile(path), nk, path)
                    for c, (path, nk) in sorted(job.swap.items())]}
     vg.run_job(oracle, env, rec, [(True, 1), (True, 10), (False, 0)],

@@ -293,3 +293,22 @@ def test_a_kernel_beyond_the_profile_is_named(tmp_path):
         assert "after the profile's last row (4 rows) it launched 'fake_kernel_saxpy'" in proc.stderr
     else:   # the scheduler had left for the rendezvous; the waiting client reports
         assert "client 0 has had a record (type" in proc.stderr, proc.stderr[-2000:]
+
+
+@pytest.mark.parametrize("async_exec", [False, True])
+def test_recorded_policy_options_on_the_fake_runtime(tmp_path, async_exec):
+    """The policy options that are not in the reference (ORION_ADMIT_OVERSIZED,
+    ORION_SLIDING_THROTTLE, with the two older ones) through the live scheduler:
+    same outputs, the options named in the log header, and the recorded run
+    replayed bit-exactly by the oracle and the native core -- the marks the
+    sliding throttle asks about are events the live host has to keep."""
+    options = {"ORION_ADMIT_OVERSIZED": "1", "ORION_SLIDING_THROTTLE": "1",
+               "ORION_RESERVE_HP_CUS": "1", "ORION_CONFINE_LONG_BE": "1"}
+    res = run_child(str(tmp_path), "orion", 2, 40, async_exec=async_exec, extra_env=options)
+    assert not any(res["alive"]) and all(res["outputs_equal"]), res
+    obs = open(os.path.join(str(tmp_path), "observations.log")).read()
+    dec = open(os.path.join(str(tmp_path), "decisions.log")).read()
+    assert obs.splitlines()[0].split(" ")[4:] == ["L1", "R1", "O1", "T1"]
+    assert dec.count("\nD ") > 100
+    assert obslog.replay(obs) == dec
+    assert jobs.native_replay(obs) == dec
