@@ -29,7 +29,8 @@ be, when the time budget (--time-budget) would not hold them:
      (`no_scheduler_baseline`: what the scheduler is for);
   5. short legs of the other two job configurations (MobileNetV2 beside
      BERT-base training; BERT-large beside three trainers), the kernel pair
-     through the scheduler, and the HIP-graph variant of the headline pair;
+     through the scheduler, and two variants of the headline pair (the client
+     replaying a HIP graph; the throttle option T1);
   6. kernel pair in this process: GEMM and triad alone and side by side per
      CU-mask size, timed with HIP events on the streams they run on;
   7. CPU baselines on this host's cores: the same requests on the PyTorch CPU
@@ -470,6 +471,15 @@ def main():
                 # policy leaves best-effort kernels no room beside it
                 "options": {"ORION_RESERVE_HP_CUS": 1}, "hp": hp_summary(cg),
                 "be": be_summary(cg)[0], "records_per_iteration": cg["num_kernels"]}
+        # The headline pair with the duration throttle letting go at its half-way
+        # mark (ORION_SLIDING_THROTTLE=1, recorded as T1): not the headline, whose
+        # decisions follow the reference's rule
+        if fits("sliding_throttle_variant", 60):
+            ct = legs.run("sliding_throttle", c3_job(short + 10), args.max_be_duration,
+                          extra_env={"ORION_SLIDING_THROTTLE": "1"})
+            out["sliding_throttle_variant"] = {
+                "options": {"ORION_SLIDING_THROTTLE": 1}, "hp": hp_summary(ct),
+                "be": be_summary(ct)[0]}
     progress.note("kernels in this process: GEMM and triad alone and side by side")
     import torch
     from orion_amd import kernel_pair as kp

@@ -36,7 +36,8 @@ void* sched_init(void);
  * reference hard-codes 80, scheduler_eval.cpp:20), ORION_RECORD_DIR (write
  * observations.log / decisions.log there), ORION_QUIET,
  * ORION_SEQUENTIAL_AS_WRITTEN, and the recorded policy options
- * ORION_CONFINE_LONG_BE, ORION_RESERVE_HP_CUS, ORION_ADMIT_OVERSIZED.
+ * ORION_CONFINE_LONG_BE, ORION_RESERVE_HP_CUS, ORION_ADMIT_OVERSIZED,
+ * ORION_SLIDING_THROTTLE.
  * `models` decides one thing: with ORION_BE_RUN_AHEAD=1 only best-effort
  * clients named "gemm_bf16" or "triad_f32" queue records ahead of their
  * dispatch (see orion_client_deferred below). */
