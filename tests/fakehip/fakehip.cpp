@@ -28,6 +28,7 @@
 #include <mutex>
 #include <thread>
 #include <vector>
+#include "fakehip_kernels.h"
 
 int gettid_cached();
 
@@ -278,6 +279,15 @@ void fake_kernel_sqadd(void** p) {
   for (int i = 0; i < n; ++i) y[i] = y[i] * y[i] + c;
 }
 
+// list.ptr[k][i] = list.ptr[k][i] * scale + list.bias for every tensor k of the
+// list;  params: FakeTensorList list (by value, several KiB), float scale
+void fake_kernel_multi(void** p) {
+  const FakeTensorList* list = (const FakeTensorList*)p[0];
+  const float scale = *(float*)p[1];
+  for (int k = 0; k < list->count; ++k)
+    for (int i = 0; i < list->n[k]; ++i) list->ptr[k][i] = list->ptr[k][i] * scale + list->bias;
+}
+
 // Argument sizes of the built-in kernels (what a real runtime reads from the
 // code object): used to deep-copy a `void** args` list into a graph kernel node
 // and to unpack a HIP_LAUNCH_PARAM_BUFFER_POINTER argument buffer.
@@ -290,13 +300,30 @@ static int fake_signature(const void* f, size_t sizes[4]) {
     sizes[0] = 8; sizes[1] = 4; sizes[2] = 4;
     return 3;
   }
+  if (f == (const void*)fake_kernel_multi) {
+    sizes[0] = sizeof(FakeTensorList); sizes[1] = 4;
+    return 2;
+  }
   return -1;
+}
+// Where each argument of `f` sits in one argument buffer: every argument at its
+// natural alignment (8 bytes for a structure).  Returns the buffer's size.
+static size_t fake_offsets(const size_t sizes[4], int count, size_t offsets[4]) {
+  size_t at = 0;
+  for (int i = 0; i < count; ++i) {
+    const size_t align = sizes[i] < 8 ? sizes[i] : 8;
+    at = (at + align - 1) / align * align;
+    offsets[i] = at;
+    at += sizes[i];
+  }
+  return at;
 }
 
 // Largest block each built-in kernel may be launched with (__launch_bounds__).
 static unsigned fake_launch_bounds(const void* f) {
   if (f == (const void*)fake_kernel_saxpy) return 256;
   if (f == (const void*)fake_kernel_sqadd) return 64;
+  if (f == (const void*)fake_kernel_multi) return 512;
   return 1024;
 }
 
@@ -315,25 +342,25 @@ static std::function<void()> bind_kernel(const void* f, void** params) {
   size_t sizes[4];
   const int count = fake_signature(f, sizes);
   if (count < 0) return nullptr;
-  auto store = std::make_shared<std::vector<unsigned char>>((size_t)count * 8);
-  for (int i = 0; i < count; ++i) memcpy(store->data() + 8 * i, params[i], sizes[i]);
-  return [f, store, count] {
+  size_t offsets[4];
+  const size_t bytes = fake_offsets(sizes, count, offsets);
+  // 8-byte units: the copies are read as pointers and structures
+  auto store = std::make_shared<std::vector<uint64_t>>((bytes + 7) / 8);
+  unsigned char* base = (unsigned char*)store->data();
+  for (int i = 0; i < count; ++i) memcpy(base + offsets[i], params[i], sizes[i]);
+  return [f, store, count, offsets_copy = std::vector<size_t>(offsets, offsets + count)] {
     void* p[4];
-    for (int i = 0; i < count; ++i) p[i] = store->data() + 8 * i;
+    for (int i = 0; i < count; ++i) p[i] = (unsigned char*)store->data() + offsets_copy[i];
     ((fake_kernel_t)f)(p);
   };
 }
 // Lays the arguments of `f` out over one argument buffer, every argument at its
 // natural alignment.
 static int unpack_buffer(const void* f, unsigned char* buffer, void* unpacked[4]) {
-  size_t sizes[4];
+  size_t sizes[4], offsets[4];
   const int count = fake_signature(f, sizes);
-  size_t at = 0;
-  for (int i = 0; i < count; ++i) {
-    at = (at + sizes[i] - 1) / sizes[i] * sizes[i];
-    unpacked[i] = buffer + at;
-    at += sizes[i];
-  }
+  fake_offsets(sizes, count, offsets);
+  for (int i = 0; i < count; ++i) unpacked[i] = buffer + offsets[i];
   return count;
 }
 static void record_later(hipEvent_t e, hipStream_t s) {
@@ -351,7 +378,7 @@ struct FakeGraph { int nodes; };
 struct FakeKernelNode {
   hipKernelNodeParams params;
   void* slots[4];
-  unsigned char storage[4][8];
+  std::vector<uint64_t> storage;   // the node's own copy of the arguments
 };
 // `held`: the kernel the node holds when the call arrives (for a new node, the
 // kernel it is being created for).  This stand-in is the pessimistic reading of
@@ -380,11 +407,14 @@ static hipError_t fake_node_set(FakeKernelNode* n, const hipKernelNodeParams* p,
     copy_sizes = held_sizes;
   }
   n->params = *p;
-  memset(n->storage, 0, sizeof n->storage);
-  for (int i = 0; i < count; ++i) n->slots[i] = n->storage[i];
+  size_t offsets[4];
+  const size_t total = fake_offsets(sizes, count, offsets);
+  n->storage.assign((total + 7) / 8, 0);
+  unsigned char* base = (unsigned char*)n->storage.data();
+  for (int i = 0; i < count; ++i) n->slots[i] = base + offsets[i];
   for (int i = 0; i < copy_count; ++i) {
     const size_t bytes = copy_sizes[i] < sizes[i] ? copy_sizes[i] : sizes[i];
-    memcpy(n->storage[i], p->kernelParams[i], bytes);
+    memcpy(n->slots[i], p->kernelParams[i], bytes);
   }
   n->params.kernelParams = n->slots;
   n->params.extra = nullptr;
@@ -795,6 +825,7 @@ const char* hipGetErrorString(hipError_t) { return "fake hip error"; }
 static const char* fake_name(const void* f) {
   if (f == (const void*)fake_kernel_saxpy) return "fake_kernel_saxpy";
   if (f == (const void*)fake_kernel_sqadd) return "fake_kernel_sqadd";
+  if (f == (const void*)fake_kernel_multi) return "fake_kernel_multi";
   return "fake_kernel";
 }
 const char* hipKernelNameRef(const hipFunction_t f) { return fake_name((const void*)f); }

@@ -20,9 +20,11 @@
 #include <vector>
 
 #include "orion_scheduler.h"
+#include "../fakehip/fakehip_kernels.h"
 
 extern "C" void fake_kernel_saxpy(void** p);
 extern "C" void fake_kernel_sqadd(void** p);
+extern "C" void fake_kernel_multi(void** p);
 extern "C" void fakehip_set_costs(long long kernel_ns, long long copy_ns);
 extern "C" long fakehip_repointed_nodes(void);
 extern "C" void orion_register_stream(void* stream);
@@ -80,13 +82,26 @@ void trimmer() {
   }
 }
 
+// Kernel k of an iteration: every fifth one scales the output through a list of
+// tensors passed by value; of the others, even ones add x, odd ones square.
+inline bool is_multi(int k) { return k % 5 == 4; }
+inline float step_of(int k, float x, float y) {
+  if (is_multi(k)) return y * 0.75f + 0.0625f;
+  return (k % 2 == 0) ? 0.5f * x + y : y * y + 0.125f;
+}
+
+// The list-of-tensors kernel through each launch form; the list lives on this
+// function's stack and is overwritten before it returns.
+struct ClientState;
+hipError_t launch_multi(ClientState& st, int form);
+
 void expected(int c, int iters, float* y) {
   float x[kN];
   for (int i = 0; i < kN; ++i) { x[i] = (float)i / kN + c; y[i] = 0.0f; }
   for (int it = 0; it < iters; ++it)
     for (int k = 0; k < g_kernels[(size_t)c]; ++k)
       for (int i = 0; i < kN; ++i)
-        y[i] = (k % 2 == 0) ? 0.5f * x[i] + y[i] : y[i] * y[i] + 0.125f;
+        y[i] = step_of(k, x[i], y[i]);
 }
 
 // What a client is made of: its buffers, the stream its calls name, and what its
@@ -104,6 +119,12 @@ struct ClientState {
 // thread: calls that name the client's stream are the client's.
 void launch_one(ClientState& st, int k, int it) {
   const int c = st.c;
+  if (is_multi(k)) {
+    if (launch_multi(st, (k + it) % 3) != hipSuccess) exit(4);
+    if (hipGetLastError() != hipSuccess) { fprintf(stderr, "client %d: stale error after a launch\n", c); exit(7); }
+    for (int i = 0; i < kN; ++i) st.want[i] = step_of(k, st.host_x[i], st.want[i]);
+    return;
+  }
   int n = kN;
   float a = 0.5f, cc = 0.125f;
   // even kernels read x through a pooled temporary: cleared by a fill, then
@@ -150,8 +171,39 @@ void launch_one(ClientState& st, int k, int it) {
   if (hipGetLastError() != hipSuccess) { fprintf(stderr, "client %d: stale error after a launch\n", c); exit(7); }
   if (temp) pool_put(c, temp);
   my_y = my_x = nullptr; my_a = my_c = -1e30f; my_n = -1;
-  for (int i = 0; i < kN; ++i)
-    st.want[i] = (k % 2 == 0) ? 0.5f * st.host_x[i] + st.want[i] : st.want[i] * st.want[i] + 0.125f;
+  for (int i = 0; i < kN; ++i) st.want[i] = step_of(k, st.host_x[i], st.want[i]);
+}
+
+hipError_t launch_multi(ClientState& st, int form) {
+  // the output as four tensors of a long list; the unused entries are poison
+  FakeTensorList list;
+  memset(&list, 0x5a, sizeof list);
+  list.count = 4;
+  list.bias = 0.0625f;
+  for (int t = 0; t < 4; ++t) { list.ptr[t] = st.y + t * (kN / 4); list.n[t] = kN / 4; }
+  float scale = 0.75f;
+  void* params[] = {&list, &scale};
+  hipError_t rc;
+  if (form == 0) {
+    rc = hipModuleLaunchKernel((hipFunction_t)fake_kernel_multi, 1, 1, 1, 64, 1, 1, 0, st.stream,
+                               params, nullptr);
+  } else if (form == 1) {
+    rc = hipLaunchKernel((void*)fake_kernel_multi, dim3(1), dim3(512), params, 0, st.stream);
+  } else {
+    struct { FakeTensorList list; float scale; } buf;
+    memcpy(&buf.list, &list, sizeof list);
+    buf.scale = scale;
+    size_t size = sizeof buf;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                     HIP_LAUNCH_PARAM_END};
+    rc = hipModuleLaunchKernel((hipFunction_t)fake_kernel_multi, 1, 1, 1, 64, 1, 1, 0, st.stream,
+                               nullptr, extra);
+    memset(&buf, 0xff, sizeof buf);
+    size = 0;
+  }
+  memset(&list, 0xff, sizeof list);
+  scale = -1e30f;
+  return rc;
 }
 
 // A thread that is no client of the scheduler and launches the second half of
