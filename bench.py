@@ -398,11 +398,26 @@ def main():
             if plain.get("runs") else [plain["p50_latency"]]
         out["hp"]["isolated_runs_p50_ms"] = [r["p50_latency"] for r in co["hp_isolated"]["runs"]] \
             if co["hp_isolated"].get("runs") else [co["hp_isolated"]["p50_latency"]]
-        # what the path costs the client when there is nothing to schedule
-        out["hp"]["path_cost_p50_ms"] = co["hp_isolated"]["p50_latency"] - plain["p50_latency"]
+        # the plain-stream client again, its thread-local accesses kept off the
+        # dynamic loader's slow path the way the library keeps a scheduled
+        # client's (ORION_PLAIN_TLS_REFRESH=1): the like-for-like baseline
+        fresh = co["hp_plain_tls_fresh_isolated"]
+        out["hp"]["plain_streams_tls_fresh_isolated_ms"] = {
+            k: fresh[f"{k}_latency"] for k in ("p50", "p95", "p99")}
+        out["hp"]["requests"]["plain_streams_tls_fresh_isolated"] = fresh.get("requests")
+        out["hp"]["plain_streams_tls_fresh_isolated_runs_p50_ms"] = \
+            [r["p50_latency"] for r in fresh["runs"]] if fresh.get("runs") else [fresh["p50_latency"]]
+        # what the path costs the client when there is nothing to schedule:
+        # against the like-for-like plain client, and against the plain client as
+        # PyTorch runs it
+        out["hp"]["path_cost_p50_ms"] = co["hp_isolated"]["p50_latency"] - fresh["p50_latency"]
+        out["hp"]["path_cost_vs_plain_as_is_p50_ms"] = \
+            co["hp_isolated"]["p50_latency"] - plain["p50_latency"]
         for p in ("p50", "p99"):
             out["hp"][f"{p}_ratio_vs_plain_streams_isolated"] = (
                 co["hp_colocated"][f"{p}_latency"] / plain[f"{p}_latency"])
+            out["hp"][f"{p}_ratio_vs_plain_streams_tls_fresh_isolated"] = (
+                co["hp_colocated"][f"{p}_latency"] / fresh[f"{p}_latency"])
         out["colocation_wall_s"] = time.time() - t0
         progress.note("replaying the recorded decisions")
         out["policy_replay"] = policy_replay(os.path.join(workdir, "c3", "colocated"))

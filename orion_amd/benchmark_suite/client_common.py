@@ -119,6 +119,12 @@ class Backend:
 
     def __init__(self):
         self.lib = fe.load_capture_library()
+        # ORION_PLAIN_TLS_REFRESH=1: a client that runs unscheduled (plain stream)
+        # gets, once per request, the same treatment scheduled clients get from
+        # the interception library: its thread-local accesses are taken off the
+        # dynamic loader's slow path (csrc/capture/tls_fresh.h).  For measuring
+        # what the scheduling path itself costs, like for like.
+        self.plain_tls_refresh = os.environ.get("ORION_PLAIN_TLS_REFRESH", "0") not in ("", "0")
 
     def block(self, it):
         """Wait until iteration ``it`` has completed on the GPU.  Under the
@@ -127,8 +133,11 @@ class Backend:
         instead, so the loop measures the same thing either way."""
         if self.lib.orion_client_index() >= 0:
             self.lib.block(it)
-        elif torch.cuda.is_available():
-            torch.cuda.current_stream().synchronize()
+        else:
+            if self.plain_tls_refresh:
+                self.lib.orion_tls_fresh_check()
+            if torch.cuda.is_available():
+                torch.cuda.current_stream().synchronize()
 
     def stop(self):
         return bool(self.lib.stop()) or UNSCHEDULED_STOP.is_set()

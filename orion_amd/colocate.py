@@ -104,8 +104,10 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
 
     ``plain_streams_too``: every repeat also runs the high-priority client alone
     on a plain stream, with no scheduler and no interception library in the
-    process (``hp_plain_isolated`` in the result): what the path itself costs
-    the client, measured in the same alternation as everything else."""
+    process (``hp_plain_isolated`` in the result), and once more with its
+    thread-local accesses kept on the loader's fast path as the library keeps a
+    scheduled client's (``hp_plain_tls_fresh_isolated``): what the path itself
+    costs the client, measured in the same alternation as everything else."""
     workdir = workdir or tempfile.mkdtemp(prefix="orion_colocate_")
     hp = job[-1]
     result = {"algo": algo, "max_be_duration_ns": max_be_duration, "workdir": workdir}
@@ -122,7 +124,7 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
             result["be_isolated"].append(
                 run_job([entry], algo, os.path.join(workdir, f"iso_be{k}"),
                         max_be_duration, env=env)[0])
-    iso_runs, co_runs, plain_runs = [], [], []
+    iso_runs, co_runs, plain_runs, plain_fresh_runs = [], [], [], []
     for rep in range(repeats):
         tag = f"_{rep}" if repeats > 1 else ""
         if plain_streams_too:
@@ -130,6 +132,13 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
             plain["kernel_file"], plain["num_kernels"] = "", 0
             plain_runs.append(run_job([plain], "streams", os.path.join(workdir, "plain_hp" + tag),
                                       max_be_duration)[0])
+            # the same, its thread-local accesses kept off the dynamic loader's
+            # slow path the way the interception library keeps a scheduled
+            # client's (csrc/capture/tls_fresh.h)
+            plain_fresh_runs.append(
+                run_job([copy.deepcopy(plain)], "streams",
+                        os.path.join(workdir, "plain_fresh_hp" + tag), max_be_duration,
+                        env={"ORION_PLAIN_TLS_REFRESH": "1"})[0])
         if not skip_isolated:
             iso_runs.append(run_job([copy.deepcopy(hp)], algo,
                                     os.path.join(workdir, "iso_hp" + tag),
@@ -143,6 +152,7 @@ def experiment(job, algo="orion", max_be_duration=100_000, workdir=None,
                                    max_be_duration, env=co_env))
     if plain_runs:
         result["hp_plain_isolated"] = pooled(plain_runs)
+        result["hp_plain_tls_fresh_isolated"] = pooled(plain_fresh_runs)
     if iso_runs:
         result["hp_isolated"] = pooled(iso_runs)
     if co_runs:

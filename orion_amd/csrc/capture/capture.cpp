@@ -10,6 +10,7 @@
 // hipExtModuleLaunchKernel / hipLaunchKernel, which are interposed here, so
 // library work is captured kernel by kernel.
 #include "capture.h"
+#include "tls_fresh.h"
 
 #include <dlfcn.h>
 #include <immintrin.h>
@@ -33,11 +34,17 @@ CaptureState g_state;
 constexpr int kNotClient = -1;
 constexpr int kUncached = -2;
 
-thread_local uint32_t tl_epoch = 0;
-thread_local int tl_client = kUncached;
+// Thread-local state of this library uses the initial-exec model: one
+// instruction per access, and never the dynamic loader's __tls_get_addr, whose
+// slow path a thread can be stuck on (tls_fresh.h).  The library is loaded at
+// program start (LD_PRELOAD), where that model always fits; loaded later, its few
+// dozen bytes come out of the loader's static surplus.
+#define ORION_TLS __attribute__((tls_model("initial-exec")))
+thread_local uint32_t tl_epoch ORION_TLS = 0;
+thread_local int tl_client ORION_TLS = kUncached;
 // Set while a client thread runs a call the scheduler granted back to it, so
 // the nested real call is not captured again.
-thread_local int tl_bypass = 0;
+thread_local int tl_bypass ORION_TLS = 0;
 
 // ORION_CALL_TIMING=1: every thread adds up the time it spends inside the
 // interposed launch and copy entry points (entry to return, the real call
@@ -48,9 +55,9 @@ const bool g_call_timing = [] {
   const char* e = getenv("ORION_CALL_TIMING");
   return e && atoi(e) != 0;
 }();
-thread_local uint64_t tl_call_ns = 0;
-thread_local uint64_t tl_call_count = 0;
-thread_local int tl_call_depth = 0;
+thread_local uint64_t tl_call_ns ORION_TLS = 0;
+thread_local uint64_t tl_call_count ORION_TLS = 0;
+thread_local int tl_call_depth ORION_TLS = 0;
 
 struct CallTimer {
   timespec t0;
@@ -145,7 +152,7 @@ struct HelperPin {
 };
 std::mutex g_helper_lock;
 std::vector<HelperPin> g_helpers;
-thread_local uint32_t tl_helper_epoch = 0;
+thread_local uint32_t tl_helper_epoch ORION_TLS = 0;
 
 void pin_helper(int client) {
   if (!g_pin.on || !g_pin.clients) return;
@@ -191,7 +198,9 @@ int lookup_thread() {
 // Which client a call belongs to: the calling thread if it is a registered
 // client thread, else the client that owns the stream the call names.
 inline int client_for_call(hipStream_t stream) {
-  if (!g_state.armed.load(std::memory_order_acquire) || tl_bypass) return kNotClient;
+  if (!g_state.armed.load(std::memory_order_acquire)) return kNotClient;
+  tls_fresh_touch();   // once per thread after each reload of the helper library
+  if (tl_bypass) return kNotClient;
   const uint32_t e = g_state.epoch.load(std::memory_order_acquire);
   if (tl_epoch != e || tl_client == kUncached) {
     tl_client = lookup_thread();
@@ -499,7 +508,21 @@ int orion_client_of_stream(void* stream) { return client_for_call((hipStream_t)s
 // While on, the calling thread's HIP calls go straight to the runtime: used by
 // a client for work that must not count as part of an iteration (building the
 // model, library auto-tuning runs whose kernel count is not reproducible).
-void orion_thread_passthrough(int on) { tl_bypass = on ? 1 : 0; }
+void orion_thread_passthrough(int on) {
+  tl_bypass = on ? 1 : 0;
+  // the end of a client's un-captured warm-up: whatever it loaded lazily (solver
+  // libraries, code objects) is in the process now
+  if (!on && g_state.armed.load(std::memory_order_acquire)) tls_fresh_check();
+}
+
+// For the scheduler thread, once per completed iteration (the reloads are left
+// to the client threads, which have time for them while they wait).
+void orion_tls_fresh_touch(void) { tls_fresh_touch(); }
+
+// The same cure for a thread that is not scheduled at all (a client on a plain
+// stream calls it once per request): lets a measurement tell what the scheduling
+// path costs from what the dynamic loader's slow path costs.
+void orion_tls_fresh_check(void) { tls_fresh_check(); }
 
 // -- control calls of the client loops (reference: intercept_temp.cpp:124-142)
 
@@ -509,6 +532,7 @@ void block(int it) {
   if (idx < 0) return;  // not armed, or not a client: nothing to wait for
   ClientChannel& ch = g_state.channels[idx];
   ch.block_calls.store((int64_t)it + 1, std::memory_order_release);
+  tls_fresh_check();    // while the GPU finishes the iteration
   unsigned spins = 0;
   while (ch.released_iters.load(std::memory_order_acquire) <= (int64_t)it) {
     if (!g_state.armed.load(std::memory_order_acquire)) return;
@@ -525,6 +549,7 @@ void block(int it) {
 int stop(void) {
   const int idx = client_for_call(nullptr);
   if (idx < 0) return 0;
+  tls_fresh_touch();
   ClientChannel& ch = g_state.channels[idx];
   const int res = ch.stop.load(std::memory_order_acquire);
   if (res) ch.stop_ack.store(1, std::memory_order_release);

@@ -274,4 +274,7 @@ void orion_capture_disarm(void);
 // way into its loop: returns once nobody is running queued records on its behalf
 // any more (see flush_channel).
 void orion_capture_enter_loop(void);
+// Keeps the calling thread's thread-local accesses on the dynamic loader's fast
+// path (capture/tls_fresh.h); the scheduler thread calls it once per iteration.
+void orion_tls_fresh_touch(void);
 }

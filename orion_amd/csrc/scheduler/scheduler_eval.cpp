@@ -327,6 +327,7 @@ class LiveHost : public PolicyHost {
     if (hipStream_t direct = ch.direct_stream.load(std::memory_order_relaxed))
       (void)hip_->hipStreamSynchronize(direct);
     ch.released_iters.store((int64_t)iteration + 1, std::memory_order_release);
+    orion_tls_fresh_touch();
     mark_slot_[(size_t)client] = -1;
     const float ms = (float)iteration_us(client) / 1000.0f;
     durations_ms_[(size_t)client].push_back(ms);

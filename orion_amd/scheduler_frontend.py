@@ -70,6 +70,8 @@ def load_capture_library(path=None):
     lib.orion_thread_time_in_calls_ns.restype = c_ulonglong
     lib.orion_thread_calls.argtypes = []
     lib.orion_thread_calls.restype = c_ulonglong
+    lib.orion_tls_fresh_check.argtypes = []
+    lib.orion_tls_fresh_check.restype = None
     lib._orion_typed = True
     return lib
 

@@ -349,8 +349,12 @@ for c in range(n_clients):
     want = expected(c, iters_done[c])
     ok_outputs.append(bool(results[c] is not None and np.array_equal(results[c], want)))
 
+_reloads, _touches = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+cap.orion_tls_fresh_stats(ctypes.byref(_reloads), ctypes.byref(_touches))
+
 print(json.dumps({
     "alive": alive, "iters_done": iters_done, "handle": handle_seen,
+    "tls_fresh": {"reloads": int(_reloads.value), "touches": int(_touches.value)},
     "deferred": [int(cap.orion_client_deferred(c)) for c in range(n_clients)],
     "submitted": [int(cap.orion_client_submitted(c)) for c in range(n_clients)],
     "holder_sets": sum(1 for k, s, t in log if k == 8),

@@ -6,6 +6,7 @@
 // (under ThreadSanitizer) no data race was reported.
 #define __HIP_PLATFORM_AMD__ 1
 #include <hip/hip_runtime_api.h>
+#include <dlfcn.h>
 #include <pthread.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -28,6 +29,7 @@ extern "C" void fake_kernel_multi(void** p);
 extern "C" void fakehip_set_costs(long long kernel_ns, long long copy_ns);
 extern "C" long fakehip_repointed_nodes(void);
 extern "C" void orion_register_stream(void* stream);
+extern "C" void orion_tls_fresh_stats(unsigned long long* reloads, unsigned long long* touches);
 
 namespace {
 
@@ -70,7 +72,15 @@ void pool_put(int c, float* t) {
 }
 
 void trimmer() {
+  // STRESS_DLOPEN names a small library that this thread keeps loading and
+  // unloading, as a framework loads code lazily: every change in the set of loaded
+  // libraries makes the interception library reload its thread-local helper while
+  // client threads are calling into it
+  const char* churn = getenv("STRESS_DLOPEN");
   while (!g_trim_stop.load()) {
+    if (churn && *churn) {
+      if (void* h = dlopen(churn, RTLD_NOW | RTLD_LOCAL)) dlclose(h);
+    }
     {
       std::lock_guard<std::mutex> hold(g_pool_lock);
       for (auto& pool : g_pool) {
@@ -386,5 +396,11 @@ int main(int argc, char** argv) {
   printf("%ld graph kernel nodes re-pointed to another kernel\n", fakehip_repointed_nodes());
   if (fakehip_repointed_nodes() != 0) bad = 1;
   if (g_done.back() != hp_iters) bad = 1;
+  if (const char* want = getenv("STRESS_EXPECT_TLS_RELOADS")) {
+    unsigned long long reloads = 0, touches = 0;
+    orion_tls_fresh_stats(&reloads, &touches);
+    printf("thread-local helper: %llu reloads, %llu calls into a fresh copy\n", reloads, touches);
+    if (reloads < (unsigned long long)atoll(want) || touches < reloads) bad = 1;
+  }
   return bad;
 }
