@@ -14,6 +14,8 @@ KERNELS_LIB = os.path.join(PKG_DIR, "liborion_kernels.so")
 POLICY_LIB = os.path.join(PKG_DIR, "liborion_policy.so")
 CAPTURE_LIB = os.path.join(PKG_DIR, "libinttemp.so")
 SCHEDULER_LIB = os.path.join(PKG_DIR, "scheduler_eval.so")
+# loaded by libinttemp.so itself, at run time (csrc/capture/tls_fresh.h)
+TLS_HELPER_LIB = os.path.join(PKG_DIR, "liborion_tlsfresh.so")
 
 
 class NativeLibraryMissing(RuntimeError):
