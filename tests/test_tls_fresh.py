@@ -62,3 +62,25 @@ def test_a_stale_thread_is_cured(tmp_path):
     # back to within a fraction of the gap
     gap = best["stale_ns"] - best["fresh_ns"]
     assert best["cured_ns"] < best["fresh_ns"] + 0.4 * gap, best
+
+
+def test_an_unscheduled_thread_can_ask_for_the_same(tmp_path):
+    """orion_tls_fresh_check(): what a plain-stream client calls once per request
+    under ORION_PLAIN_TLS_REFRESH=1 (benchmark_suite/client_common.py Backend)."""
+    code = (
+        "import ctypes, json, sys\n"
+        f"sys.path.insert(0, {ROOT!r})\n"
+        "from orion_amd import scheduler_frontend as fe\n"
+        "lib = fe.load_capture_library()\n"
+        "r, t = ctypes.c_ulonglong(), ctypes.c_ulonglong()\n"
+        "lib.orion_tls_fresh_stats(ctypes.byref(r), ctypes.byref(t)); before = (r.value, t.value)\n"
+        "lib.orion_tls_fresh_check(); lib.orion_tls_fresh_check()\n"
+        "lib.orion_tls_fresh_stats(ctypes.byref(r), ctypes.byref(t))\n"
+        "print(json.dumps({'before': before, 'after': (r.value, t.value)}))\n")
+    env = dict(os.environ, ORION_HIP_LIBRARY=os.path.join(ROOT, "tests", "fakehip", "libfakehip.so"))
+    out = subprocess.run([os.sys.executable, "-c", code], check=True, capture_output=True,
+                         text=True, env=env, timeout=120).stdout
+    res = json.loads(out.strip().splitlines()[-1])
+    assert res["before"] == [0, 0]
+    # one reload (nothing was loaded between the two calls), one call into it
+    assert res["after"] == [1, 1], res
