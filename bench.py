@@ -21,8 +21,11 @@ the GPU when it starts them); legs after the headline are skipped, and said to
 be, when the time budget (--time-budget) would not hold them:
   1. profile both clients alone under the interception layer (gfx950 profiles);
   2. best-effort client alone; then, alternating --repeats times: the
-     high-priority client alone on a plain stream with no library in the process,
-     alone behind the interception layer and the scheduler, and co-located;
+     high-priority client alone on a plain stream with the interception library
+     not preloaded (once as PyTorch runs it, once with its thread-local accesses
+     kept on the dynamic loader's fast path as the library keeps a scheduled
+     client's: the like-for-like baseline), alone behind the interception layer
+     and the scheduler, and co-located;
   3. replay the recorded observation log through the CPU oracle and the native
      policy core: decision sequences must be identical;
   4. the same pair on plain streams with no scheduler and no interception
@@ -378,10 +381,11 @@ def main():
 
     if not args.kernels_only:
         t0 = time.time()
-        # every repeat: the client alone on a plain stream (no library in the
-        # process), alone behind the interception layer and the scheduler, and
-        # co-located -- so that what the path costs and what co-location costs are
-        # differences inside one alternation, not between boxes or minutes
+        # every repeat: the client alone on a plain stream (the library not
+        # preloaded; as it is and with the thread-local cure), alone behind the
+        # interception layer and the scheduler, and co-located -- so that what the
+        # path costs and what co-location costs are differences inside one
+        # alternation, not between boxes or minutes
         co = legs.run("c3", c3_job(per_run + 10), args.max_be_duration, repeats=repeats,
                       use_rocprof=args.rocprof_profiles, record=True, plain_streams_too=True)
         out["value"] = co["hp_p99_ratio"]

@@ -147,6 +147,14 @@ class Backend:
         entry points (0 unless ORION_CALL_TIMING=1)."""
         return int(self.lib.orion_thread_time_in_calls_ns())
 
+    def tls_fresh_stats(self):
+        """Reloads of the thread-local helper library in this process so far, and
+        calls of threads into a fresh copy (csrc/capture/tls_fresh.h)."""
+        import ctypes
+        reloads, touches = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        self.lib.orion_tls_fresh_stats(ctypes.byref(reloads), ctypes.byref(touches))
+        return {"reloads": int(reloads.value), "touches": int(touches.value)}
+
     def register_stream(self, stream):
         self.lib.orion_register_stream(stream.cuda_stream)
 
@@ -255,6 +263,8 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
     if extra:
         data.update(extra())
     data["iterations"] = batch_idx
+    if hasattr(backend, "tls_fresh_stats"):
+        data["tls_fresh"] = backend.tls_fresh_stats()
     if not train:
         # every measured request, in arrival order (the reference's file holds
         # the percentiles only): lets runs be pooled

@@ -72,6 +72,8 @@ def load_capture_library(path=None):
     lib.orion_thread_calls.restype = c_ulonglong
     lib.orion_tls_fresh_check.argtypes = []
     lib.orion_tls_fresh_check.restype = None
+    lib.orion_tls_fresh_stats.argtypes = [POINTER(c_ulonglong), POINTER(c_ulonglong)]
+    lib.orion_tls_fresh_stats.restype = None
     lib._orion_typed = True
     return lib
 
