@@ -105,9 +105,13 @@ void tls_fresh_touch_slow() {
   if (touch_fn fn = g_touch.load(std::memory_order_seq_cst)) {
     fn();
     g_touches.fetch_add(1, std::memory_order_relaxed);
-    tl_tls_fresh_seen = count;   // a reload in between brings the thread back here
   }
   g_users.fetch_sub(1, std::memory_order_release);
+  // Also when there was nothing to call (a reload is under way, or the helper
+  // library could not be loaded): the reload counter moves on when a reload
+  // completes and brings the thread back here; until then it stays off the
+  // shared counters above.
+  tl_tls_fresh_seen = count;
 }
 
 void tls_fresh_check() {

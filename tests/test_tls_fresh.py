@@ -84,3 +84,11 @@ def test_an_unscheduled_thread_can_ask_for_the_same(tmp_path):
     assert res["before"] == [0, 0]
     # one reload (nothing was loaded between the two calls), one call into it
     assert res["after"] == [1, 1], res
+
+
+def test_a_missing_helper_library_is_reported_once_and_nothing_else_changes(tmp_path):
+    proc_env = {"ORION_TLS_REFRESH_LIBRARY": str(tmp_path / "no_such_library.so")}
+    res = run_child(str(tmp_path), "orion", 1, 20, extra_env=proc_env)
+    assert all(res["outputs_equal"]), res
+    assert res["iters_done"][-1] == 20
+    assert res["tls_fresh"]["touches"] == 0 and res["tls_fresh"]["reloads"] >= 1
