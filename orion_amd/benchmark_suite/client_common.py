@@ -151,8 +151,11 @@ class Backend:
         """Reloads of the thread-local helper library in this process so far, and
         calls of threads into a fresh copy (csrc/capture/tls_fresh.h)."""
         import ctypes
+        lib = getattr(self, "lib", None)
+        if lib is None:
+            return None
         reloads, touches = ctypes.c_ulonglong(), ctypes.c_ulonglong()
-        self.lib.orion_tls_fresh_stats(ctypes.byref(reloads), ctypes.byref(touches))
+        lib.orion_tls_fresh_stats(ctypes.byref(reloads), ctypes.byref(touches))
         return {"reloads": int(reloads.value), "touches": int(touches.value)}
 
     def register_stream(self, stream):
@@ -263,8 +266,9 @@ def run_client(tid, train, num_iters, sleep_times, barriers, step, backend,
     if extra:
         data.update(extra())
     data["iterations"] = batch_idx
-    if hasattr(backend, "tls_fresh_stats"):
-        data["tls_fresh"] = backend.tls_fresh_stats()
+    fresh = backend.tls_fresh_stats() if hasattr(backend, "tls_fresh_stats") else None
+    if fresh is not None:
+        data["tls_fresh"] = fresh
     if not train:
         # every measured request, in arrival order (the reference's file holds
         # the percentiles only): lets runs be pooled

@@ -36,19 +36,16 @@ def test_capture_and_scheduler_are_race_free(tmp_path):
     subprocess.run(common + srcs + [os.path.join(ROOT, "tests", "native", "stress_capture.cpp"),
                                     fake, "-Wl,-rpath," + str(tmp_path), "-ldl", "-o", exe],
                    check=True)
-    # the thread-local helper library, and a second small library that the stress
-    # program keeps loading and unloading so that the helper is reloaded while
-    # client threads call into it
+    # the thread-local helper library is loaded once here; reloading it while
+    # clients run is left to the un-sanitized run below (the sanitizer's own
+    # bookkeeping of dynamically allocated thread-local blocks does not survive a
+    # library being unloaded and loaded again: it aborts inside its
+    # __tls_get_addr interceptor, not in the code under test)
     helper = str(tmp_path / "liborion_tlsfresh.so")
     subprocess.run(["gcc", "-O2", "-fPIC", "-ftls-model=global-dynamic", "-shared",
                     os.path.join(CSRC, "capture", "tls_fresh_helper.c"), "-o", helper], check=True)
-    churn_src = tmp_path / "churn.c"
-    churn_src.write_text("static __thread long v;\nlong churn_touch(void) { return ++v; }\n")
-    churn = str(tmp_path / "libchurn.so")
-    subprocess.run(["gcc", "-O2", "-fPIC", "-shared", str(churn_src), "-o", churn], check=True)
     env = dict(os.environ, ORION_HIP_LIBRARY=fake, ORION_QUIET="1",
-               ORION_TLS_REFRESH_LIBRARY=helper, STRESS_DLOPEN=churn,
-               STRESS_EXPECT_TLS_RELOADS="2",
+               ORION_TLS_REFRESH_LIBRARY=helper, STRESS_EXPECT_TLS_RELOADS="1",
                TSAN_OPTIONS="halt_on_error=1 exitcode=66 second_deadlock_stack=1")
     env.pop("LD_PRELOAD", None)
     # both hand-offs of the high-priority client: issuing its own calls and
@@ -92,7 +89,19 @@ def test_order_and_lifetime_on_the_asynchronous_runtime(tmp_path):
     subprocess.run(common + srcs + [os.path.join(ROOT, "tests", "native", "stress_capture.cpp"),
                                     fake, "-Wl,-rpath," + str(tmp_path), "-ldl", "-o", exe],
                    check=True)
-    env = dict(os.environ, ORION_HIP_LIBRARY=fake, ORION_QUIET="1", FAKEHIP_ASYNC="1")
+    # a small library with thread-local storage that the stress program keeps
+    # loading and unloading, so that the interception library reloads its helper
+    # every few milliseconds while client threads are calling into it
+    helper = str(tmp_path / "liborion_tlsfresh.so")
+    subprocess.run(["gcc", "-O2", "-fPIC", "-ftls-model=global-dynamic", "-shared",
+                    os.path.join(CSRC, "capture", "tls_fresh_helper.c"), "-o", helper], check=True)
+    churn_src = tmp_path / "churn.c"
+    churn_src.write_text("static __thread long v;\nlong churn_touch(void) { return ++v; }\n")
+    churn = str(tmp_path / "libchurn.so")
+    subprocess.run(["gcc", "-O2", "-fPIC", "-shared", str(churn_src), "-o", churn], check=True)
+    env = dict(os.environ, ORION_HIP_LIBRARY=fake, ORION_QUIET="1", FAKEHIP_ASYNC="1",
+               ORION_TLS_REFRESH_LIBRARY=helper, STRESS_DLOPEN=churn,
+               STRESS_EXPECT_TLS_RELOADS="2")
     env.pop("LD_PRELOAD", None)
     for seed in range(4):
         for clients, ahead in ((3, "0"), (3, "1"), (4, "1")):
