@@ -108,11 +108,12 @@ int orion_client_index(void);
  * for; negative when the call would go straight to the runtime (reference
  * counterpart of the lookup: get_idx, src/cuda_capture/utils_interc.cpp:3-51). */
 int orion_client_of_stream(void* stream);
-/* The CPU the calling client or scheduler thread was pinned to when it was
- * first identified (reference: the sched_setaffinity of get_idx,
- * src/cuda_capture/utils_interc.cpp:36-49), or -1 when it is not pinned
- * (ORION_PIN_THREADS=0, too few CPUs, not a client).  The masks in force
- * before are restored when the job ends. */
+/* With ORION_PIN_THREADS=1: the CPU the calling client or scheduler thread was
+ * pinned to when it was first identified (reference: the sched_setaffinity of
+ * get_idx, src/cuda_capture/utils_interc.cpp:36-49).  -1 when it is not pinned:
+ * by default (threads are left to the kernel's placement, which measured
+ * better on the hosts of these GPUs), with too few CPUs, or for a thread that
+ * is no client.  The masks in force before are restored when the job ends. */
 int orion_pinned_cpu(void);
 
 /* No reference counterpart: while on, the calling thread's HIP calls bypass the

@@ -4,6 +4,7 @@ scheduler's own thread and strangers pass through).  Here the lookup is cached
 per thread, and calls from unregistered threads (autograd workers) are routed by
 the stream they name.  Runs in a child process: arming is process-global."""
 
+import os
 import subprocess
 import sys
 import textwrap
@@ -71,7 +72,8 @@ CHILD = textwrap.dedent("""
 
 def test_thread_and_stream_identity():
     out = subprocess.run([sys.executable, "-c", CHILD, _lib.CAPTURE_LIB],
-                         capture_output=True, text=True, timeout=60)
+                         capture_output=True, text=True, timeout=60,
+                         env=dict(os.environ, ORION_PIN_THREADS="1"))
     assert out.returncode == 0, out.stderr
     seen = dict(eval(out.stdout.strip().splitlines()[-1]))
     for i in range(3):
