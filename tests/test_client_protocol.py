@@ -268,3 +268,49 @@ def test_queueing_ahead_is_refused_for_framework_trainers(monkeypatch):
     monkeypatch.setenv("ORION_BE_RUN_AHEAD_UNSAFE", "1")
     with pytest.raises(RuntimeError, match="gemm_bf16, triad_f32"):
         lj.job_lists(trainer_pair)
+
+
+def test_the_experiment_alternates_plain_isolated_and_colocated_runs(tmp_path, monkeypatch):
+    """colocate.experiment with plain_streams_too: every repeat runs the
+    high-priority client on a plain stream as it is, on a plain stream with the
+    thread-local cure, alone through the library, and co-located -- in that
+    order, so that the four are compared inside one alternation."""
+    from orion_amd import colocate
+    calls = []
+
+    def fake_run_job(job, algo, workdir, max_be_duration, env=None, **kw):
+        calls.append((os.path.basename(workdir), algo, len(job), dict(env or {})))
+        out = []
+        for k, entry in enumerate(job):
+            res = {"throughput": 10.0 + k}
+            if not entry["args"]["train"]:
+                lat = [1.0 + 0.01 * len(calls)] * 20
+                res.update({"p50_latency": lat[0], "p95_latency": lat[0], "p99_latency": lat[0],
+                            "latencies_ms": lat})
+            out.append(res)
+        return out
+
+    monkeypatch.setattr(colocate, "run_job", fake_run_job)
+    job = [{"arch": "x", "kernel_file": "be.csv", "num_kernels": 3, "num_iters": 100,
+            "args": {"train": True}},
+           {"arch": "x", "kernel_file": "hp.csv", "num_kernels": 5, "num_iters": 30,
+            "args": {"train": False}}]
+    res = colocate.experiment(job, workdir=str(tmp_path), repeats=2, plain_streams_too=True,
+                              env={"ORION_RECORD_DIR": str(tmp_path / "rec")})
+    names = [c[0] for c in calls]
+    assert names == ["iso_be0",
+                     "plain_hp_0", "plain_fresh_hp_0", "iso_hp_0", "colocated_0",
+                     "plain_hp_1", "plain_fresh_hp_1", "iso_hp_1", "colocated_1"]
+    by_name = {c[0]: c for c in calls}
+    assert by_name["plain_hp_0"][1] == "streams" and by_name["plain_hp_0"][3] == {}
+    assert by_name["plain_fresh_hp_1"][1] == "streams"
+    assert by_name["plain_fresh_hp_1"][3] == {"ORION_PLAIN_TLS_REFRESH": "1"}
+    assert by_name["iso_hp_0"][1] == "orion" and by_name["colocated_0"][2] == 2
+    # only the last co-located run keeps the recorded logs
+    assert "ORION_RECORD_DIR" not in by_name["colocated_0"][3]
+    assert by_name["colocated_1"][3]["ORION_RECORD_DIR"] == str(tmp_path / "rec")
+    for key in ("hp_plain_isolated", "hp_plain_tls_fresh_isolated", "hp_isolated", "hp_colocated"):
+        assert res[key]["requests"] == 40, key
+    assert res["hp_p99_ratio"] == pytest.approx(
+        res["hp_colocated"]["p99_latency"] / res["hp_isolated"]["p99_latency"])
+    assert res["be_retained"] == [1.0]
