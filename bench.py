@@ -330,8 +330,9 @@ def main():
                     help="skip every leg after the headline, its replay, the kernels and "
                          "the headline's CPU baseline")
     ap.add_argument("--short-requests", type=int, default=400,
-                    help="measured high-priority requests of the short legs (other job "
-                         "configurations, HIP-graph variant)")
+                    help="measured high-priority requests of the short legs (HIP-graph and "
+                         "throttle variants; MobileNetV2 beside BERT training runs twice, "
+                         "BERT-large beside three trainers five times as many)")
     ap.add_argument("--pair-requests", type=int, default=300,
                     help="measured GEMM requests of the scheduled kernel pair")
     ap.add_argument("--repeats", type=int, default=4,
@@ -435,13 +436,15 @@ def main():
         short = args.short_requests
         # configs[3] and configs[4], short: a p99 over `short` requests is a few
         # samples deep; the parity tests of these configurations are in tests/
-        if fits("c4_mobilenet_beside_bert_base_training", 90):
-            c4 = legs.run("c4", c4_job(short + 10), 100_000)
+        # (twice and five times `short`: their request rates are higher, so the
+        # legs stay a few seconds long while the p99 gets 8 and 20 samples deep)
+        if fits("c4_mobilenet_beside_bert_base_training", 100):
+            c4 = legs.run("c4", c4_job(2 * short + 10), 100_000)
             out["c4_mobilenet_beside_bert_base_training"] = {
                 "workload": "configs[3], budget 100 us", "hp": hp_summary(c4), "be": be_summary(c4),
                 "records_per_iteration": c4["num_kernels"]}
-        if fits("c5_bert_large_beside_three_trainers", 150):
-            c5 = legs.run("c5", c5_job(short + 50), 100_000)
+        if fits("c5_bert_large_beside_three_trainers", 170):
+            c5 = legs.run("c5", c5_job(5 * short + 50), 100_000)
             out["c5_bert_large_beside_three_trainers"] = {
                 "workload": "configs[4], budget 100 us, closed loop", "hp": hp_summary(c5),
                 "be": be_summary(c5), "records_per_iteration": c5["num_kernels"]}
