@@ -118,6 +118,11 @@ def test_resnet50_colocation_outputs_and_replay(tmp_path):
                           160000, env={"ORION_SAVE_OUTPUT_DIR": co_dir,
                                        "ORION_RECORD_DIR": co_dir})
     assert co[-1]["iterations"] == 40 and co[0]["iterations"] >= 10
+    # the thread-local helper library was found beside libinttemp.so, reloaded
+    # after the clients' lazy loading, and called by both client threads and the
+    # scheduler thread (csrc/capture/tls_fresh.h); no reload storm
+    fresh = co[-1]["tls_fresh"]
+    assert 1 <= fresh["reloads"] <= 20 and fresh["touches"] >= 3, fresh
     iso_out = torch.load(os.path.join(iso_dir, "client_0_output.pt"), weights_only=True)
     co_out = torch.load(os.path.join(co_dir, "client_1_output.pt"), weights_only=True)
     # Same kernels, deterministic solvers: bit-exact.  (Without the
