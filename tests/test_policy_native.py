@@ -32,6 +32,57 @@ def test_orion_inference_hp(tmp_path, seed, n_clients):
     assert oracle.cur_iters[-1] == 25
 
 
+@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("n_clients", [2, 3])
+def test_a_cu_budget_of_one_holds_best_effort_kernels_while_a_request_is_in_flight(
+        tmp_path, seed, n_clients):
+    """max_sms = 1 (ORION_MAX_SMS=1, the setting for inference beside inference):
+    the CU clause ``size + sm_used <= max_sms`` (scheduler_eval.cpp:339-340) can
+    admit no kernel that needs more than one CU, so while a high-priority request
+    is in flight (``seen[hp] > 0``) no such best-effort kernel is dispatched;
+    between requests they go at once (:333).  Oracle and native core agree bit
+    for bit, and the rule is checked decision by decision on the oracle's log."""
+    from tests.test_policy_properties import check_orion_invariants
+
+    def held_kernels(max_sms):
+        work = tmp_path / str(max_sms)
+        work.mkdir()
+        job = jobs.make_job(str(work), seed=400 + seed, n_clients=n_clients, max_sms=max_sms,
+                            hp_iters=200)
+        # the reference's rule alone (the random job may have drawn an option)
+        job.admit_oversized = job.sliding_throttle = False
+        job.reserve_hp = job.confine_long = False
+        oracle, env, rec = jobs.run_oracle(job)
+        marked = jobs.native_replay(rec.obs_text(), by_poll=True)
+        assert "".join(l + "\n" for l in marked.splitlines() if l != "P") == rec.dec.text()
+        # the reference's per-poll rules, re-stated on the logs, at this budget
+        check_orion_invariants(rec.obs_text(), marked, job.depth)
+        hp = n_clients - 1
+        in_flight, done, during, between = False, [0] * n_clients, 0, 0
+        for line in rec.dec.text().splitlines():
+            f = line.split(" ")
+            if f[0] == "D" and f[3] == "k":
+                client = int(f[1])
+                if client == hp:
+                    in_flight = True
+                elif (done[client] > 10 and done[hp] < oracle.max_iters[hp]      # past :335
+                      and oracle.ops[client][int(f[4])].sm_used > 1):
+                    during += in_flight
+                    between += not in_flight
+            elif f[0] == "F":
+                done[int(f[1])] += 1
+                if int(f[1]) == hp:
+                    in_flight = False
+            elif f[0] == "S":           # a new call of schedule(): iterations count from 0
+                in_flight, done = False, [0] * n_clients
+        return during, between
+
+    during_1, between_1 = held_kernels(1)
+    during_256, _ = held_kernels(256)
+    assert during_1 == 0 and between_1 > 5
+    assert during_256 > 0        # the same job under the device's budget admits some
+
+
 @pytest.mark.parametrize("seed", range(8))
 @pytest.mark.parametrize("n_clients", [2, 3])
 def test_orion_training_hp(tmp_path, seed, n_clients):
