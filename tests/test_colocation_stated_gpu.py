@@ -23,7 +23,8 @@ of the network's depth, the *_RTOL values below: one and a half times what was
 measured on an MI355X -- 7.7e-3 (ResNet-50; 5.1e-3 with deterministic solvers),
 2.6e-2 (MobileNetV2, whose depthwise layers have short accumulations that do
 not average the roundings out) and 3.4e-2 (BERT-large, 24 layers) -- and
-measured values are printed into gpurun_out/ when that directory exists.  Between the isolated and the
+measured values are appended to a file in the directory ORION_TEST_REPORT_DIR
+names, when it is set.  Between the isolated and the
 co-located run of the same bf16 client only the order of atomic accumulations
 can differ (split-K convolution and GEMM solvers).  configs[2] and configs[3]
 therefore run twice: with the libraries' default solvers -- the kernels bench.py
@@ -114,8 +115,9 @@ def _run(work, job, budget, profiles, be_alone=()):
 
 
 def _report(name, **values):
-    if os.path.isdir("gpurun_out"):
-        with open(os.path.join("gpurun_out", "stated_configs_errors.jsonl"), "a") as f:
+    report_dir = os.environ.get("ORION_TEST_REPORT_DIR")
+    if report_dir and os.path.isdir(report_dir):
+        with open(os.path.join(report_dir, "stated_configs_errors.jsonl"), "a") as f:
             f.write(json.dumps({"config": name, **values}) + "\n")
 
 

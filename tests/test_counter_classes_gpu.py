@@ -47,6 +47,7 @@ def test_triad_and_gemm_classes_from_counters_alone(tmp_path):
             assert fam["memory_fraction"] > 0.5 > fam["valu_fraction"] and fam["mfma_fraction"] == 0
         else:             # the GEMM keeps the matrix cores busy
             assert fam["mfma_fraction"] > 0.5 > fam["memory_fraction"]
-        if os.path.isdir("gpurun_out"):
-            with open(os.path.join("gpurun_out", "counter_classes.jsonl"), "a") as f:
+        report_dir = os.environ.get("ORION_TEST_REPORT_DIR")
+        if report_dir and os.path.isdir(report_dir):
+            with open(os.path.join(report_dir, "counter_classes.jsonl"), "a") as f:
                 f.write(json.dumps({"client": entry["arch"], "kernel": name, **fam, **stats}) + "\n")
