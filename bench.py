@@ -229,6 +229,54 @@ def policy_replay(record_dir):
     }
 
 
+def own_children():
+    """Process ids whose parent is this process (threads are not processes)."""
+    me, found = os.getpid(), []
+    for name in os.listdir("/proc"):
+        if not name.isdigit():
+            continue
+        try:
+            with open(f"/proc/{name}/stat") as f:
+                stat = f.read()
+            # pid (comm) state ppid ...: comm may hold spaces and parentheses
+            ppid = int(stat[stat.rindex(")") + 2:].split()[1])
+        except (OSError, ValueError, IndexError):
+            continue
+        if ppid == me:
+            found.append(int(name))
+    return found
+
+
+def end_own_children(grace_s=2.0):
+    """Ends child processes that are still alive, each by its own process id:
+    first asked to terminate, then killed.  Returns how many there were."""
+    import signal
+    children = own_children()
+    found = len(children)
+    for pid in children:
+        try:
+            os.kill(pid, signal.SIGTERM)
+        except OSError:
+            pass
+    deadline = time.time() + grace_s
+    while children and time.time() < deadline:
+        for pid in list(children):
+            try:
+                done, _ = os.waitpid(pid, os.WNOHANG)
+            except ChildProcessError:
+                done = pid
+            if done:
+                children.remove(pid)
+        time.sleep(0.05)
+    for pid in children:
+        try:
+            os.kill(pid, signal.SIGKILL)
+            os.waitpid(pid, 0)
+        except OSError:
+            pass
+    return found
+
+
 def host_cores():
     """Threads the CPU baselines use: the CPUs this process may run on, capped by
     OMP_NUM_THREADS when the environment sets one (a shared host hands out a
@@ -563,6 +611,9 @@ def main():
     if not others:
         skipped.append("cpu_baseline.others")
     out["skipped"] = skipped
+    # every leg waits for the children it started; whatever is still there now
+    # (there should be nothing) is ended here, by process id, and counted
+    out["children_ended_at_exit"] = end_own_children()
     out["wall_s"] = time.time() - t_start
     print(json.dumps(out))
     return 0
