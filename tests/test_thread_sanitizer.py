@@ -109,3 +109,46 @@ def test_order_and_lifetime_on_the_asynchronous_runtime(tmp_path):
                                   env=dict(env, ORION_BE_RUN_AHEAD=ahead, FAKEHIP_SEED=str(seed + 1)),
                                   capture_output=True, text=True, timeout=600)
             assert proc.returncode == 0, (seed, clients, ahead, proc.stdout + proc.stderr[-4000:])
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_capture_and_scheduler_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """The same stress program with AddressSanitizer and UBSan (host code only),
+    the thread-local helper being reloaded under churn while clients run: a record
+    read after its slot was reused, an argument copy past its buffer or a call into
+    an unloaded helper copy would be reported here."""
+    exe = str(tmp_path / "stress_asan")
+    fake = str(tmp_path / "libfakehip_asan.so")
+    common = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
+              "-fno-omit-frame-pointer", "-fPIC", "-pthread",
+              "-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include",
+              "-I" + os.path.join(CSRC, "policy")]
+    subprocess.run(common + ["-shared", os.path.join(ROOT, "tests", "fakehip", "fakehip.cpp"),
+                             "-o", fake], check=True)
+    srcs = [os.path.join(CSRC, p) for p in (
+        "capture/capture.cpp", "capture/tls_fresh.cpp", "common/hip_api.cpp", "policy/policy.cpp",
+        "policy/obslog.cpp",
+        "scheduler/scheduler_eval.cpp", "scheduler/profile_capture.cpp")]
+    subprocess.run(common + srcs + [os.path.join(ROOT, "tests", "native", "stress_capture.cpp"),
+                                    fake, "-Wl,-rpath," + str(tmp_path), "-ldl", "-o", exe],
+                   check=True)
+    helper = str(tmp_path / "liborion_tlsfresh.so")
+    subprocess.run(["gcc", "-O2", "-fPIC", "-ftls-model=global-dynamic", "-shared",
+                    os.path.join(CSRC, "capture", "tls_fresh_helper.c"), "-o", helper], check=True)
+    churn_src = tmp_path / "churn.c"
+    churn_src.write_text("static __thread long v;\nlong churn_touch(void) { return ++v; }\n")
+    churn = str(tmp_path / "libchurn.so")
+    subprocess.run(["gcc", "-O2", "-fPIC", "-shared", str(churn_src), "-o", churn], check=True)
+    env = dict(os.environ, ORION_HIP_LIBRARY=fake, ORION_QUIET="1",
+               ORION_TLS_REFRESH_LIBRARY=helper, STRESS_DLOPEN=churn,
+               STRESS_EXPECT_TLS_RELOADS="2",
+               ASAN_OPTIONS="detect_leaks=0 abort_on_error=0 exitcode=67",
+               UBSAN_OPTIONS="halt_on_error=1 exitcode=68 print_stacktrace=1")
+    env.pop("LD_PRELOAD", None)
+    for clients, ahead, later in ((3, "1", "0"), (4, "1", "1"), (3, "0", "1")):
+        proc = subprocess.run([exe, str(tmp_path), str(clients), "40"],
+                              env=dict(env, ORION_BE_RUN_AHEAD=ahead, FAKEHIP_ASYNC=later),
+                              capture_output=True, text=True, timeout=600)
+        assert "ERROR: AddressSanitizer" not in proc.stderr, proc.stderr[-4000:]
+        assert "runtime error:" not in proc.stderr, proc.stderr[-4000:]
+        assert proc.returncode == 0, proc.stdout + proc.stderr[-4000:]
