@@ -21,7 +21,8 @@ req/s on average); pass it with ``--hp-trace`` to do the same.
 
     python -m orion_amd.figures --figure 7 --out fig7 [--pairs rnet_rnet bert_mnet]
         [--algo orion|reef|sequential|streams] [--hp-hip-graph]
-        [--env ORION_RESERVE_HP_CUS=1 ...] [--hp-trace inter_arrival_times.json]
+        [--env ORION_RESERVE_HP_CUS=1 ...] [--budget-scale 2.5]
+        [--hp-trace inter_arrival_times.json]
 """
 
 import argparse
@@ -107,10 +108,12 @@ def markdown(rows, figure):
 
 def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
         experiment=None, fill_job=None, log=print, algo="orion", hp_hip_graph=False,
-        env=None):
+        env=None, budget_scale=1.0):
     """``algo``: ``orion``, ``reef`` (depth 12), ``sequential``, or ``streams`` -- the
     same clients on plain streams with no scheduler, the reference's "Streams"
-    baseline; it needs no profiles."""
+    baseline; it needs no profiles.  ``budget_scale`` multiplies every pair's
+    duration budget (the reference's own per-pair figures were chosen on a
+    V100)."""
     from . import colocate
     from .profiling import capture_profile
     experiment = experiment or colocate.experiment
@@ -128,6 +131,7 @@ def run(figure, out_dir, pairs=None, hp_requests=1200, repeats=2, hp_trace=None,
         for name, (job, budget) in todo.items():
             if pairs and name not in pairs:
                 continue
+            budget = int(round(budget * budget_scale))
             base = os.path.join(out_dir, name)
             os.makedirs(base, exist_ok=True)
             cfg = os.path.join(base, "job.json")
@@ -166,11 +170,14 @@ def main(argv=None):
                    help="the high-priority client replays a captured HIP graph per request")
     p.add_argument("--env", nargs="*", default=[], metavar="KEY=VALUE",
                    help="environment of every run, e.g. ORION_MAX_SMS=8")
+    p.add_argument("--budget-scale", type=float, default=1.0,
+                   help="multiply every pair's duration budget (1.0 = the reference's own)")
     p.add_argument("--hp-trace", help="JSON list of inter-arrival times (s) for the "
                                       "high-priority client instead of Poisson arrivals")
     a = p.parse_args(argv)
     rows = run(a.figure, a.out, a.pairs, a.hp_requests, a.repeats, a.hp_trace, algo=a.algo,
-               hp_hip_graph=a.hp_hip_graph, env=dict(kv.split("=", 1) for kv in a.env))
+               hp_hip_graph=a.hp_hip_graph, env=dict(kv.split("=", 1) for kv in a.env),
+               budget_scale=a.budget_scale)
     print(markdown(rows, a.figure))
 
 

@@ -80,6 +80,13 @@ def test_driver_writes_one_row_per_pair(tmp_path):
     assert rows[0]["pair"] == "rnet_rnet"
     with pytest.raises(KeyError):
         figures.run(7, str(tmp_path), pairs=["nope"], experiment=experiment, fill_job=fill_job)
+    # every pair's budget scaled (the reference's own figures were chosen on a V100)
+    del seen[:]
+    figures.run(7, str(tmp_path / "scaled"), pairs=["bert_mnet", "rnet_rnet"], hp_requests=400,
+                repeats=2, experiment=experiment, fill_job=fill_job, log=lambda *_: None,
+                budget_scale=2.5)
+    assert [s[2] for s in seen] == [400_000, 250_000]
+    assert "| rnet_rnet | 400 µs |" in open(tmp_path / "scaled" / "fig7.md").read()
 
 
 def test_hip_graph_and_other_policies_are_options_of_the_same_pairs(tmp_path):
